@@ -1,0 +1,226 @@
+/* C ABI of the MI355X host-staged expert-dispatch runtime.
+ *
+ * This is the drop-in boundary for the reference's native extension: every
+ * entry point below names the reference interface it replaces (paths relative
+ * to the reference checkout).  Signatures use plain pointers and sizes only;
+ * device pointers are ordinary HIP device addresses and `stream` is a
+ * `hipStream_t` passed as `void*`.
+ *
+ * Error convention: functions returning `int` return 0 on success and a
+ * negative `PCIE_EP_E_*` code otherwise; `pcie_ep_last_error()` then holds a
+ * message whose text mirrors the reference's `TORCH_CHECK` messages so that a
+ * binding can raise the same exception types.  Device-side protocol errors are
+ * never reported here: they land in the `errors[8]` output array with the
+ * reference's numeric codes (csrc/kernels/host_staged/common.cuh:26-38).
+ */
+#ifndef PCIE_EP_AMD_H
+#define PCIE_EP_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCIE_EP_ABI_VERSION 1
+
+#define PCIE_EP_E_INVALID (-1)   /* bad argument / unsupported dimensions (ValueError / RuntimeError) */
+#define PCIE_EP_E_HIP (-2)       /* a HIP runtime call failed */
+#define PCIE_EP_E_STATE (-3)     /* runtime closed, or call not legal in this state */
+#define PCIE_EP_E_TIMEOUT (-4)   /* a host-side wait timed out */
+#define PCIE_EP_E_PROTOCOL (-5)  /* the host peer emulator observed a protocol violation */
+
+typedef struct pcie_ep_runtime pcie_ep_runtime;
+
+/* Replaces the (directory, rank, p, t, h, k, e, options) constructor arguments
+ * of AdvancedRuntime (csrc/buffers/advanced.hpp:107) and the option dict parsed
+ * by AdvancedConfig (csrc/comm/advanced_shared_memory.hpp:55-112). */
+typedef struct pcie_ep_config {
+    int32_t num_ranks;          /* P logical ranks, 1..16 */
+    int32_t local_rank;         /* the rank this GPU plays */
+    int32_t max_tokens;         /* num_max_tokens_per_rank */
+    int32_t hidden;
+    int32_t topk;               /* 1..32 */
+    int32_t num_experts;        /* divisible by num_ranks, <= 4096 */
+    int32_t channels;           /* 1..32 */
+    int32_t payload_slots;      /* Q per channel */
+    int32_t descriptor_slots;   /* L per (channel, destination) */
+    int32_t wire_fp8;           /* 0 BF16 wire, 1 E4M3FN + FP32 scale per token */
+    int32_t timeout_ms;         /* device-side protocol timeout */
+    int32_t fuse_receive_expand;/* 1: receive waves scatter to expert rows; 0: unique rows + expand kernel */
+    int32_t tx_waves;           /* payload TX wavefronts per channel, 0 = default */
+    int32_t rx_waves;           /* payload RX wavefronts per channel, 0 = default */
+    int32_t peer_threads;       /* host threads standing in for the other ranks; 0 = none */
+    int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
+    int32_t device;             /* HIP device ordinal */
+    int32_t reserved[7];
+} pcie_ep_config;
+
+/* Capacities and byte sizes a caller needs to allocate pools
+ * (csrc/buffers/advanced.hpp:296-326, :21-41). */
+typedef struct pcie_ep_sizes {
+    int64_t unique_rows;        /* P * Tmax */
+    int64_t expanded_rows;      /* unique_rows * min(K, E/P) + (E/P) * 255 */
+    int64_t plan_bytes;         /* one route-plan blob */
+    int64_t segment_bytes;      /* one pinned source segment */
+    int64_t slot_stride;        /* bytes between payload slots */
+    int32_t local_experts;
+    int32_t payload_bytes;      /* wire bytes of one row */
+    int32_t meta_bytes;         /* per-slot token metadata bytes */
+    int32_t mailbox_dwords;
+    int32_t transport_threads;  /* workgroup size of the transport kernel */
+    int32_t reserved[7];
+} pcie_ep_sizes;
+
+/* One dispatch: inputs, the route plan to fill or reuse, and every output of
+ * one result pool.  Field-for-field the tensors AdvancedRuntime binds in
+ * bind_state (csrc/buffers/advanced.hpp:420-470).  All pointers are device
+ * pointers that stay valid until the stream has executed the dispatch. */
+typedef struct pcie_ep_dispatch_args {
+    const void* x;                   /* bf16 [T, H] */
+    const int64_t* topk_idx;         /* [T, K] global expert ids, -1 unused */
+    const float* topk_weights;       /* [T, K] or NULL */
+    int32_t num_tokens;              /* T <= max_tokens */
+    int32_t alignment;               /* 1..256 */
+    int32_t expand;                  /* do_expand */
+    int32_t zero_padding;
+    int32_t reuse_plan;              /* 1: `plan` already holds this routing (cached layout) */
+    int32_t reserved0;
+    void* plan;                      /* plan_bytes */
+    void* unique_payload;            /* bf16 [unique_rows, H] */
+    int64_t* unique_topk_idx;        /* [unique_rows, K] */
+    float* unique_topk_weights;      /* [unique_rows, K] */
+    int64_t* unique_source_meta;     /* [unique_rows, 3] */
+    int32_t* unique_expert_ordinals; /* [unique_rows, K] */
+    void* expanded_payload;          /* bf16 [expanded_rows, H] */
+    int64_t* expanded_expert_idx;    /* [expanded_rows] */
+    float* expanded_weights;         /* [expanded_rows] */
+    int64_t* expanded_source_meta;   /* [expanded_rows, 3] */
+    int64_t* unique_count;           /* [1] */
+    int64_t* expanded_count;         /* [1] */
+    int32_t* expert_prefix;          /* [E/P] */
+    int32_t* expert_counts;          /* [E/P] */
+    int32_t* expert_offsets;         /* [E/P + 1] */
+    int32_t* source_offsets;         /* [P + 1] */
+    int32_t* source_expert_prefix;   /* [P, E/P] */
+    int64_t* errors;                 /* [8] */
+    int64_t* stats;                  /* [8] */
+    int64_t* transport_timestamps_ns;/* [2] */
+    int32_t* expected_receive_counts;/* [C, P] */
+    int64_t* channel_stats;          /* [C, 8] */
+    int64_t* channel_timestamps_ns;  /* [C, 2] */
+    int64_t* receive_expand_overlap; /* [C, 2] */
+    uint64_t* receive_prefix_state;  /* [2] */
+    int64_t* prefix_tx_timestamps_ns;/* [C + 1, 2] */
+    int64_t expanded_capacity_rows;  /* rows actually allocated for expanded_* */
+} pcie_ep_dispatch_args;
+
+int pcie_ep_abi_version(void);
+
+/* Pure host arithmetic, usable without a GPU.  Replaces the capacity formulas
+ * of allocate_workspace (advanced.hpp:296-298) and the segment size of
+ * make_advanced_shared_memory_layout (advanced_common.cuh:42-84). */
+int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes);
+
+/* Replaces create_advanced_segments + prepare_advanced_segment +
+ * AdvancedRuntime::AdvancedRuntime (csrc/comm/advanced_shared_memory.hpp:143-212,
+ * csrc/buffers/advanced.hpp:107-124): allocates and zeroes the P pinned
+ * fine-grained host segments, the device workspace and, when
+ * `peer_threads > 0`, the host peer emulator. */
+int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** runtime);
+
+/* Replaces AdvancedRuntime::close (advanced.hpp:229-240).  The caller must have
+ * synchronised every stream that ran a dispatch. */
+int pcie_ep_runtime_destroy(pcie_ep_runtime* runtime);
+
+/* Replaces AdvancedRuntime::dispatch / launch_dispatch (advanced.hpp:126-156,
+ * :472-523): enqueues the dispatch kernels on `stream`, never synchronises and
+ * never allocates, so it may be called under stream capture. */
+int pcie_ep_dispatch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
+
+/* Thread-local message of the last failing call (runtime may be NULL). */
+const char* pcie_ep_last_error(void);
+
+/* Test-only hooks (advanced.hpp:158-180; csrc/runtime.cu:23-27). */
+int pcie_ep_set_test_delays(pcie_ep_runtime* runtime, uint64_t metadata_ns, uint64_t tx_ns, uint64_t rx_ns, uint64_t scatter_ns);
+int pcie_ep_set_test_prefix_delay_ns(pcie_ep_runtime* runtime, uint64_t delay_ns);
+int pcie_ep_set_test_control_abort_after_ns(pcie_ep_runtime* runtime, uint64_t delay_ns);
+int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* runtime, int32_t source);
+
+/* Replaces get_device_numa_node (advanced_shared_memory.hpp:120-131). */
+int pcie_ep_device_numa_node(int32_t device);
+
+/* Host-visible protocol words, for failure tests that force a condition from
+ * the CPU (the reference's destructor does the same store: advanced.hpp:258-261).
+ * which: 0 abort, 1 channel_abort[index], 2 counts_ready, 3 counts_consumed[index]. */
+int pcie_ep_host_signal_store(pcie_ep_runtime* runtime, int32_t segment_rank, int32_t which, int32_t index, uint64_t value);
+int pcie_ep_host_signal_load(pcie_ep_runtime* runtime, int32_t segment_rank, int32_t which, int32_t index, uint64_t* value);
+
+/* ---- Stand-alone kernels (same device code the dispatch uses) ------------ */
+
+/* Replaces quantize_transport_payload (csrc/kernels/host_staged/quantization.cuh:34-71):
+ * bf16 [T,H] -> E4M3FN codes [T,H] + FP32 scale [T]. */
+int pcie_ep_quantize_fp8(const void* x, uint8_t* codes, float* scales, int32_t tokens, int32_t hidden, void* stream);
+/* Replaces dequantize_fp8_to_bf16 (quantization.cuh:21-24) over whole rows. */
+int pcie_ep_dequantize_fp8(const uint8_t* codes, const float* scales, void* out, int32_t tokens, int32_t hidden, void* stream);
+/* Replaces scatter_expert_inputs (csrc/kernels/host_staged/dispatch.cuh:8-65): expands
+ * the unique rows of `args` into its expert-major outputs using the prefixes
+ * already present in `args` (what a non-fused dispatch launches last). */
+int pcie_ep_expand_unique(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
+
+/* Pinned-copy bandwidth of this box (GB/s, best of `repeats`), the denominator
+ * for "% of x16 peak".  No counterpart in the reference. */
+int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, double* h2d_gbps, double* d2h_gbps);
+
+/* ---- Host peer emulator ---------------------------------------------------
+ * On one GPU the other logical ranks are host threads that follow the ring
+ * protocol on the same pinned segments, the way the reference's CPU relay
+ * workers do (csrc/comm/numa_relay.hpp:18-35, :240-340).  As sources they stage
+ * payload, metadata, descriptors and counts for rows destined to the GPU's
+ * rank; as receivers they consume the GPU's descriptors, optionally capture
+ * the rows, and return ACKs and credits. */
+
+/* Give rank `rank` (!= local_rank) its inputs for the following epochs; host
+ * pointers, copied.  `weights` may be NULL (1.0 is sent, as the reference does:
+ * advanced_dispatch.cuh:73).  tokens may be 0. */
+int pcie_ep_peer_set_source(pcie_ep_runtime* runtime, int32_t rank, const void* x_bf16, const int64_t* topk_idx,
+                            const float* weights, int32_t tokens);
+/* Serve the next `epochs` dispatches. flags bit 0: capture rows received from the GPU. */
+int pcie_ep_peers_start(pcie_ep_runtime* runtime, int32_t epochs, uint32_t flags);
+/* Block until every emulated source has staged all it can for the first
+ * pending epoch without GPU progress (used to pre-stage before timing). */
+int pcie_ep_peers_wait_staged(pcie_ep_runtime* runtime, int32_t timeout_ms);
+/* Block until all started epochs are served; returns PCIE_EP_E_PROTOCOL /
+ * PCIE_EP_E_TIMEOUT with a message on failure. */
+int pcie_ep_peers_wait(pcie_ep_runtime* runtime, int32_t timeout_ms);
+/* Abandon outstanding epochs (after a GPU-side failure). */
+int pcie_ep_peers_cancel(pcie_ep_runtime* runtime);
+/* Rows rank `rank` received from the GPU in the last served epoch: count, then
+ * copies (row order = arrival order per channel; `tokens[i]` identifies the row).
+ * payload is wire bytes [count, payload_bytes]; idx/ordinals/weights are [count, K]. */
+int pcie_ep_peer_captured_count(pcie_ep_runtime* runtime, int32_t rank, int64_t* count);
+int pcie_ep_peer_captured_copy(pcie_ep_runtime* runtime, int32_t rank, int32_t* tokens, int32_t* rank_ordinals,
+                               uint8_t* payload, float* scales, int32_t* expert_idx, int32_t* expert_ordinals,
+                               float* weights, uint32_t* destination_masks);
+/* Force a protocol failure from the host.  fault: 1 withhold counts_ready,
+ * 2 withhold counts_consumed, 3 withhold the last payload ACK, 4 publish a
+ * wrong payload sequence.  Applies to rank `rank` for the next started epochs;
+ * fault 0 clears. */
+int pcie_ep_peers_inject_fault(pcie_ep_runtime* runtime, int32_t rank, int32_t fault);
+
+/* Host implementations the emulator uses, exposed so CPU tests can check them
+ * against the oracle without a GPU. */
+int pcie_ep_host_quantize_fp8(const void* x_bf16, uint8_t* codes, float* scales, int32_t tokens, int32_t hidden);
+int pcie_ep_host_dequantize_fp8(const uint8_t* codes, const float* scales, void* out_bf16, int32_t tokens, int32_t hidden);
+/* Route plan of one source on the host: mask [T], rank_ordinals [T,P],
+ * expert_indices [T,K], expert_ordinals [T,K], counts [P+E]; returns 0, or 2
+ * (the device error code) for invalid routing. */
+int pcie_ep_host_source_layout(const int64_t* topk_idx, int32_t tokens, int32_t topk, int32_t num_ranks, int32_t num_experts,
+                               uint32_t* mask, int32_t* rank_ordinals, int32_t* expert_indices, int32_t* expert_ordinals,
+                               int32_t* counts);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCIE_EP_AMD_H */

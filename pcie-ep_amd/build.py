@@ -1,0 +1,71 @@
+"""Build the gfx950 shared library in-tree.
+
+    python pcie-ep_amd/build.py            # compile every source, link the .so
+    python pcie-ep_amd/build.py --if-missing
+
+hipcc cross-compiles for gfx950 without a GPU.  The library lands in
+``pcie-ep_amd/pcie_ep/lib/libpcie_ep_amd.so`` so it travels with the tree.
+"""
+
+from __future__ import annotations
+
+import argparse
+import concurrent.futures
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+OUT_DIR = HERE / "pcie_ep" / "lib"
+LIBRARY = OUT_DIR / "libpcie_ep_amd.so"
+OBJ_DIR = HERE / "build"
+
+HIP_SOURCES = ["prologue_kernel.hip", "transport_kernel.hip", "expand_kernels.hip", "runtime.hip"]
+CXX_SOURCES = ["peers.cpp"]
+
+COMMON = ["-O3", "-std=c++20", "-fPIC", "-Wall", "-Wno-unused-function", "-pthread"]
+# Packed FP32 instructions are disabled for all device code of this build.
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(command: list[str]) -> None:
+    result = subprocess.run(command, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    stderr = "\n".join(line for line in result.stderr.splitlines() if noise not in line)
+    if result.returncode != 0:
+        raise RuntimeError(f"{' '.join(command)}\n{result.stdout}\n{stderr}")
+    if stderr.strip():
+        print(stderr, file=sys.stderr)
+
+
+def _compile(name: str) -> Path:
+    source = CSRC / name
+    target = OBJ_DIR / (name + ".o")
+    command = ["hipcc", *COMMON]
+    if name.endswith(".hip"):
+        command += DEVICE
+    command += ["-c", str(source), "-o", str(target)]
+    _run(command)
+    return target
+
+
+def build(force: bool = True) -> Path:
+    if not force and LIBRARY.exists():
+        return LIBRARY
+    if shutil.which("hipcc") is None:
+        raise RuntimeError("hipcc not found: the HIP extension cannot be built")
+    OBJ_DIR.mkdir(exist_ok=True)
+    OUT_DIR.mkdir(exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
+        objects = list(pool.map(_compile, HIP_SOURCES + CXX_SOURCES))
+    _run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-pthread", *map(str, objects), "-o", str(LIBRARY)])
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--if-missing", action="store_true")
+    arguments = parser.parse_args()
+    print(build(force=not arguments.if_missing))

@@ -1,0 +1,235 @@
+// Device-side state, synchronisation primitives and wavefront row movers for
+// the gfx950 dispatch kernels.  Wave size is 64 throughout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "fp8.h"
+#include "wire.h"
+
+namespace pcie_ep {
+
+constexpr int kWave = 64;
+constexpr uint64_t kTicksPerUs = 100;  // wall_clock64() runs at 100 MHz on gfx950
+constexpr uint64_t kPrefixFailed = ~uint64_t(0);
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Launch argument of every kernel: this rank's device pointers, the device
+// aliases of the pinned host segments and the plan/output pool of one dispatch
+// (the role of AdvancedDeviceState: csrc/kernels/host_staged/advanced_common.cuh:86-129).
+struct DeviceState {
+    SegmentLayout z;
+    char* seg[kMaxRanks];
+    int local_rank;
+    int tx_waves;
+    int rx_waves;
+    int fuse_expand;  // receive waves scatter straight into expert rows
+    int expand;
+    int alignment;
+    int num_tokens;
+    int zero_padding;
+    int reuse_plan;
+    int counts_ack_skip_source;
+    uint64_t timeout_ticks;
+    uint64_t* epoch;
+
+    const uint16_t* x;
+    const int64_t* topk_idx;
+    const float* topk_weights;
+
+    // Route plan (immutable once built; a cached layout pins it).
+    uint32_t* plan_mask;      // [Tmax]
+    int32_t* plan_rank_ord;   // [Tmax, P]
+    int32_t* plan_exp_idx;    // [Tmax, K]
+    int32_t* plan_exp_ord;    // [Tmax, K]
+    int32_t* plan_counts;     // [P + E]
+    int32_t* plan_chan_counts;// [C, P]
+    int32_t* plan_chan_remote;// [C]
+
+    int32_t* chan_remote_tokens;  // scratch [C, ceil(Tmax / C)]: ring history for slot reuse
+
+    uint16_t* unique_payload;
+    int64_t* unique_topk_idx;
+    float* unique_topk_weights;
+    int64_t* unique_source_meta;
+    int32_t* unique_expert_ordinals;
+    uint16_t* expanded_payload;
+    int64_t* expanded_expert_idx;
+    float* expanded_weights;
+    int64_t* expanded_source_meta;
+    int64_t expanded_capacity;
+    int64_t* unique_count;
+    int64_t* expanded_count;
+    int32_t* expert_prefix;
+    int32_t* expert_counts;
+    int32_t* expert_offsets;
+    int32_t* source_offsets;
+    int32_t* source_expert_prefix;
+    int64_t* errors;
+    int64_t* stats;
+    int64_t* transport_timestamps_ns;
+    int32_t* expected_receive_counts;
+    int64_t* channel_stats;
+    int64_t* channel_timestamps_ns;
+    int64_t* receive_expand_overlap;
+    uint64_t* receive_prefix_state;
+    int64_t* prefix_tx_timestamps_ns;
+
+    // Test hooks, in clock ticks (advanced_common.cuh:118-124).
+    uint64_t metadata_delay;
+    uint64_t tx_delay;
+    uint64_t rx_delay;
+    uint64_t scatter_delay;
+    uint64_t prefix_delay;
+    uint64_t control_abort_after;
+};
+
+// ---- clocks and back-off ---------------------------------------------------
+
+__device__ __forceinline__ uint64_t now_ticks() { return wall_clock64(); }
+__device__ __forceinline__ int64_t ticks_to_ns(uint64_t ticks) { return int64_t(ticks * (1000 / kTicksPerUs)); }
+__device__ __forceinline__ void backoff() { __builtin_amdgcn_s_sleep(8); }
+
+__device__ inline void test_delay(uint64_t ticks) {
+    if (!ticks) return;
+    const uint64_t start = now_ticks();
+    while (now_ticks() - start < ticks) __builtin_amdgcn_s_sleep(16);
+}
+
+// ---- system-scope signals on pinned host memory ------------------------------
+
+__device__ __forceinline__ uint64_t load_acquire_system(const uint64_t* address) {
+    return __hip_atomic_load(address, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ uint64_t load_relaxed_system(const uint64_t* address) {
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void store_release_system(uint64_t* address, uint64_t value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void fence_acquire_system() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
+__device__ __forceinline__ void fence_release_system() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
+
+// ---- workgroup-scope hand-off through LDS -----------------------------------
+
+__device__ __forceinline__ int lds_load(const int* address) {
+    return __hip_atomic_load(address, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_store(int* address, int value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void fence_workgroup() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); }
+
+// ---- device-scope flags in HBM -----------------------------------------------
+
+__device__ __forceinline__ uint64_t load_acquire_device(const uint64_t* address) {
+    return __hip_atomic_load(address, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_release_device(uint64_t* address, uint64_t value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int64_t load_error_code(const DeviceState& state) {
+    return __hip_atomic_load(state.errors, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// First error wins; context fields follow the reference
+// (advanced_common.cuh:289-295: errors[1] = local rank, errors[2] = epoch).
+__device__ inline void record_error(const DeviceState& state, int code, int64_t context = -1, int64_t detail = -1) {
+    unsigned long long expected = 0;
+    if (atomicCAS(reinterpret_cast<unsigned long long*>(state.errors), expected, static_cast<unsigned long long>(code)) == 0ull) {
+        state.errors[1] = context >= 0 ? context : state.local_rank;
+        state.errors[2] = detail >= 0 ? detail : int64_t(*state.epoch);
+    }
+}
+
+// ---- lane helpers ---------------------------------------------------------------
+
+__device__ __forceinline__ int lane_id() { return int(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
+__device__ __forceinline__ uint64_t lanes_below(int lane) { return lane >= 64 ? ~0ull : ((1ull << lane) - 1ull); }
+__device__ __forceinline__ int broadcast_first(int value) { return __builtin_amdgcn_readfirstlane(value); }
+
+// ---- abort flags on the host segments ----------------------------------------------
+// Flags per rank: abort, then channel_abort[C].  All 64 lanes load in parallel
+// (the reference scans 32 at a time: advanced_common.cuh:350-378).
+__device__ inline bool any_abort_wave(const DeviceState& state, int lane) {
+    const int per_rank = 1 + state.z.dims.channels;
+    const int flags = state.z.dims.num_ranks * per_rank;
+    bool aborted = false;
+    for (int index = lane; index < flags; index += kWave) {
+        char* segment = state.seg[index / per_rank];
+        const int flag = index % per_rank;
+        const uint64_t* signal = flag == 0 ? signal_at(segment, state.z.abort_offset)
+                                           : signal_at(segment, state.z.channel_abort_offset, flag - 1);
+        aborted |= load_acquire_system(signal) != 0;
+    }
+    return __any(aborted);
+}
+
+// Bounded failure detection: the local timeout is checked on every call, the
+// remote flags at most every min(1 ms, timeout / 8) (advanced_common.cuh:380-429).
+struct HealthCheck {
+    uint64_t start;
+    uint64_t next_scan;
+    uint64_t interval;
+    __device__ HealthCheck(const DeviceState& state, uint64_t begin) : start(begin) {
+        const uint64_t cap = 1000 * kTicksPerUs;
+        const uint64_t eighth = state.timeout_ticks / 8;
+        interval = eighth < cap ? eighth : cap;
+        next_scan = begin + interval;
+    }
+    __device__ bool poll(const DeviceState& state, int lane) {
+        const uint64_t now = now_ticks();
+        if (now - start > state.timeout_ticks) return true;
+        // `now` differs slightly per lane; take lane 0's verdict for the scan.
+        const int scan = broadcast_first(now >= next_scan ? 1 : 0);
+        if (!scan) return false;
+        const bool failed = any_abort_wave(state, lane);
+        next_scan = now_ticks() + interval;
+        return failed;
+    }
+};
+
+// ---- wavefront row movers ----------------------------------------------------------
+// One wavefront moves a whole row: every lane keeps up to kPassItems 16-byte
+// vectors in registers, all loads of a pass are issued before the first use,
+// so a 14 336-byte BF16 row is 14 loads in flight per lane and is read once
+// however many expert rows it is scattered to.
+constexpr int kPassItems = 16;
+
+struct RowVectors {
+    u32x4 v[kPassItems];
+};
+
+// Vector index of item j for this lane: j * 64 + lane (consecutive lanes touch
+// consecutive 16-byte vectors: 1 KiB contiguous per instruction).
+template <bool kNonTemporal>
+__device__ __forceinline__ void row_load_vectors(RowVectors& row, const u32x4* source, int first, int count, int lane) {
+#pragma unroll
+    for (int j = 0; j < kPassItems; ++j) {
+        const int index = first + j * kWave + lane;
+        if (index < count) row.v[j] = kNonTemporal ? __builtin_nontemporal_load(source + index) : source[index];
+    }
+}
+template <bool kNonTemporal>
+__device__ __forceinline__ void row_store_vectors(const RowVectors& row, u32x4* destination, int first, int count, int lane) {
+#pragma unroll
+    for (int j = 0; j < kPassItems; ++j) {
+        const int index = first + j * kWave + lane;
+        if (index < count) {
+            if (kNonTemporal) __builtin_nontemporal_store(row.v[j], destination + index);
+            else destination[index] = row.v[j];
+        }
+    }
+}
+
+// Scalar fall-back for rows whose byte length is not a multiple of 16: the
+// same structure with 2-byte items (the reference also falls back to scalar
+// copies for such hidden sizes: csrc/kernels/host_staged/fused_receive.cuh:116-126).
+constexpr int kPassScalars = 32;
+struct RowScalars {
+    uint16_t v[kPassScalars];
+};
+
+}  // namespace pcie_ep

@@ -1,0 +1,116 @@
+// Whole-row helpers executed by one 64-lane wavefront: plain copy, FP8 wire
+// quantisation (per-token amax -> scale -> E4M3FN codes) and de-quantisation.
+// The quantiser restates quantize_transport_payload of the reference
+// (csrc/kernels/host_staged/quantization.cuh:34-71) for one wavefront per token.
+#pragma once
+
+#include "device_common.h"
+
+namespace pcie_ep {
+
+__device__ __forceinline__ float wave_max(float value) {
+    for (int offset = 32; offset > 0; offset >>= 1) value = fmaxf(value, __shfl_xor(value, offset));
+    return value;
+}
+
+// BF16 row copy.  kVector requires hidden % 8 == 0 and 16-byte aligned rows.
+template <bool kVector, bool kStreamOut>
+__device__ inline void copy_row(const uint16_t* input, uint16_t* output, int hidden, int lane) {
+    if constexpr (kVector) {
+        const int vectors = hidden / 8;
+        const u32x4* source = reinterpret_cast<const u32x4*>(input);
+        u32x4* destination = reinterpret_cast<u32x4*>(output);
+        for (int first = 0; first < vectors; first += kPassItems * kWave) {
+            RowVectors row;
+            row_load_vectors<true>(row, source, first, vectors, lane);
+            row_store_vectors<kStreamOut>(row, destination, first, vectors, lane);
+        }
+    } else {
+        for (int index = lane; index < hidden; index += kWave) output[index] = input[index];
+    }
+}
+
+// Returns the row scale.  kVector requires hidden % 16 == 0.
+template <bool kVector>
+__device__ inline float quantize_row(const uint16_t* input, uint8_t* output, int hidden, int lane) {
+    // Sweep 1: row amax in FP32.  Sweep 2 re-reads the row (it is L2 resident).
+    float amax = 0.0f;
+    if constexpr (kVector) {
+        const int vectors = hidden / 8;
+        const u32x4* source = reinterpret_cast<const u32x4*>(input);
+        for (int index = lane; index < vectors; index += kWave) {
+            const u32x4 v = source[index];
+#pragma unroll
+            for (int word = 0; word < 4; ++word) {
+                amax = fmaxf(amax, fabsf(bf16_to_float(uint16_t(v[word] & 0xFFFFu))));
+                amax = fmaxf(amax, fabsf(bf16_to_float(uint16_t(v[word] >> 16))));
+            }
+        }
+    } else {
+        for (int index = lane; index < hidden; index += kWave) amax = fmaxf(amax, fabsf(bf16_to_float(input[index])));
+    }
+    amax = wave_max(amax);
+    const float scale = fp8_scale_from_amax(amax);
+    // Multiply by the correctly rounded FP32 reciprocal, as the reference does
+    // (quantization.cuh:66; pcie_ep/quantization.py:27-29), not a division per element.
+    const float inverse = 1.0f / scale;
+    if constexpr (kVector) {
+        // 16 elements (two 16-byte loads) -> 16 codes (one 16-byte store) per lane.
+        const int groups = hidden / 16;
+        const u32x4* source = reinterpret_cast<const u32x4*>(input);
+        u32x4* destination = reinterpret_cast<u32x4*>(output);
+        for (int group = lane; group < groups; group += kWave) {
+            const u32x4 lo = source[group * 2], hi = source[group * 2 + 1];
+            u32x4 codes;
+#pragma unroll
+            for (int word = 0; word < 4; ++word) {
+                const uint32_t a = word < 2 ? lo[word * 2] : hi[(word - 2) * 2];
+                const uint32_t b = word < 2 ? lo[word * 2 + 1] : hi[(word - 2) * 2 + 1];
+                codes[word] = uint32_t(fp8_quantize_element(uint16_t(a & 0xFFFFu), inverse)) |
+                              uint32_t(fp8_quantize_element(uint16_t(a >> 16), inverse)) << 8 |
+                              uint32_t(fp8_quantize_element(uint16_t(b & 0xFFFFu), inverse)) << 16 |
+                              uint32_t(fp8_quantize_element(uint16_t(b >> 16), inverse)) << 24;
+            }
+            destination[group] = codes;
+        }
+    } else {
+        for (int index = lane; index < hidden; index += kWave) output[index] = fp8_quantize_element(input[index], inverse);
+    }
+    return scale;
+}
+
+// 16 codes -> two 16-byte vectors of BF16 (elements in order).
+__device__ __forceinline__ void dequantize_vector(const u32x4& codes, float scale, u32x4& lo, u32x4& hi) {
+#pragma unroll
+    for (int word = 0; word < 4; ++word) {
+        const uint32_t c = codes[word];
+        const uint32_t a = uint32_t(fp8_dequantize_element(uint8_t(c), scale)) | uint32_t(fp8_dequantize_element(uint8_t(c >> 8), scale)) << 16;
+        const uint32_t b = uint32_t(fp8_dequantize_element(uint8_t(c >> 16), scale)) | uint32_t(fp8_dequantize_element(uint8_t(c >> 24), scale)) << 16;
+        if (word < 2) {
+            lo[word * 2] = a;
+            lo[word * 2 + 1] = b;
+        } else {
+            hi[(word - 2) * 2] = a;
+            hi[(word - 2) * 2 + 1] = b;
+        }
+    }
+}
+
+template <bool kVector>
+__device__ inline void dequantize_row(const uint8_t* codes, float scale, uint16_t* output, int hidden, int lane) {
+    if constexpr (kVector) {
+        const int groups = hidden / 16;
+        const u32x4* source = reinterpret_cast<const u32x4*>(codes);
+        u32x4* destination = reinterpret_cast<u32x4*>(output);
+        for (int group = lane; group < groups; group += kWave) {
+            u32x4 lo, hi;
+            dequantize_vector(source[group], scale, lo, hi);
+            destination[group * 2] = lo;
+            destination[group * 2 + 1] = hi;
+        }
+    } else {
+        for (int index = lane; index < hidden; index += kWave) output[index] = fp8_dequantize_element(codes[index], scale);
+    }
+}
+
+}  // namespace pcie_ep

@@ -1,0 +1,515 @@
+// Host side of the runtime and its C ABI (include/pcie_ep_amd.h).
+//
+// Replaces the host half of the reference's native extension: AdvancedRuntime
+// (csrc/buffers/advanced.hpp:44-552), the segment creation / first touch /
+// registration helpers (csrc/comm/advanced_shared_memory.hpp:143-288) and the
+// pybind module (csrc/runtime.cu:8-29).  Tensor allocation and pool ownership
+// live in the caller; this library owns the pinned segments, a few KB of device
+// workspace and the host peer emulator.
+#include <hip/hip_runtime.h>
+
+#include <linux/mempolicy.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include <cctype>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <memory>
+#include <string>
+
+#include "../../include/pcie_ep_amd.h"
+#include "launch.h"
+#include "peers.h"
+
+using namespace pcie_ep;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int set_error(int code, const char* format, ...) {
+    char buffer[1024];
+    va_list arguments;
+    va_start(arguments, format);
+    vsnprintf(buffer, sizeof buffer, format, arguments);
+    va_end(arguments);
+    g_last_error = buffer;
+    return code;
+}
+
+#define HIP_TRY(expression)                                                                                   \
+    do {                                                                                                      \
+        hipError_t status_ = (expression);                                                                    \
+        if (status_ != hipSuccess)                                                                            \
+            return set_error(PCIE_EP_E_HIP, "%s failed: %s", #expression, hipGetErrorString(status_));        \
+    } while (0)
+
+// Plan blob sub-layout (the tensors of AdvancedLayout: advanced.hpp:21-41).
+struct PlanLayout {
+    size_t mask, rank_ord, exp_idx, exp_ord, counts, chan_counts, chan_remote, bytes;
+};
+
+PlanLayout plan_layout(const Dimensions& d) {
+    PlanLayout p{};
+    size_t cursor = 0;
+    auto reserve = [&](size_t bytes) {
+        const size_t offset = cursor;
+        cursor += align_up(bytes, 256);
+        return offset;
+    };
+    const size_t tokens = size_t(d.max_tokens);
+    p.mask = reserve(tokens * 4);
+    p.rank_ord = reserve(tokens * d.num_ranks * 4);
+    p.exp_idx = reserve(tokens * d.topk * 4);
+    p.exp_ord = reserve(tokens * d.topk * 4);
+    p.counts = reserve(size_t(d.num_ranks + d.num_experts) * 4);
+    p.chan_counts = reserve(size_t(d.channels) * d.num_ranks * 4);
+    p.chan_remote = reserve(size_t(d.channels) * 4);
+    p.bytes = cursor;
+    return p;
+}
+
+int check_config(const pcie_ep_config* c, Dimensions& dims) {
+    if (!c) return set_error(PCIE_EP_E_INVALID, "config is NULL");
+    // advanced.hpp:110-112
+    if (!(c->num_ranks >= 1 && c->num_ranks <= kMaxRanks && c->local_rank >= 0 && c->local_rank < c->num_ranks && c->max_tokens > 0 &&
+          c->hidden > 0 && c->topk > 0 && c->topk <= kMaxTopk && c->num_experts >= c->num_ranks && c->num_experts <= kMaxExperts &&
+          c->num_experts % c->num_ranks == 0))
+        return set_error(PCIE_EP_E_INVALID, "unsupported advanced dimensions");
+    // advanced_shared_memory.hpp:106-111
+    if (c->channels < 1 || c->channels > kMaxChannels) return set_error(PCIE_EP_E_INVALID, "channels must be 1..32");
+    if (c->payload_slots <= 0 || c->descriptor_slots <= 0 || c->timeout_ms <= 0)
+        return set_error(PCIE_EP_E_INVALID, "invalid advanced capacity or timeout");
+    if (c->tx_waves < 0 || c->tx_waves > kMaxTxWaves || c->rx_waves < 0 || c->rx_waves > kMaxRxWaves)
+        return set_error(PCIE_EP_E_INVALID, "tx_waves must be 0..%d and rx_waves 0..%d", kMaxTxWaves, kMaxRxWaves);
+    if (c->peer_threads < 0) return set_error(PCIE_EP_E_INVALID, "peer_threads must be non-negative");
+    dims = Dimensions{c->num_ranks, c->max_tokens, c->hidden, c->topk, c->num_experts, c->channels, c->payload_slots, c->descriptor_slots,
+                      c->wire_fp8 ? 1 : 0};
+    return 0;
+}
+
+}  // namespace
+
+struct pcie_ep_runtime {
+    pcie_ep_config config{};
+    SegmentLayout z{};
+    PlanLayout plan{};
+    char* segments[kMaxRanks] = {};
+    uint64_t* epoch = nullptr;
+    int32_t* chan_remote_tokens = nullptr;
+    int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves;
+    uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
+    int counts_ack_skip_source = -1;
+    std::unique_ptr<PeerEmulator> peers;
+    bool closed = false;
+};
+
+namespace {
+
+uint64_t ns_to_ticks(uint64_t ns) { return ns / (1000 / kTicksPerUs); }
+
+int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState& s) {
+    const Dimensions& d = rt->z.dims;
+    if (rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!a) return set_error(PCIE_EP_E_INVALID, "dispatch args are NULL");
+    // advanced.hpp:367-380
+    if (a->num_tokens < 0 || a->num_tokens > d.max_tokens || (a->num_tokens > 0 && (!a->x || !a->topk_idx)))
+        return set_error(PCIE_EP_E_INVALID, "bad advanced input");
+    if (a->alignment < 1 || a->alignment > 256) return set_error(PCIE_EP_E_INVALID, "alignment must be in [1,256]");
+    if (!a->plan) return set_error(PCIE_EP_E_INVALID, "route plan storage is NULL");
+    if (a->zero_padding && !a->expand) return set_error(PCIE_EP_E_INVALID, "zero padding requires expand");
+    const void* required[] = {a->unique_payload, a->unique_topk_idx, a->unique_topk_weights, a->unique_source_meta, a->unique_expert_ordinals,
+                              a->expanded_payload, a->expanded_expert_idx, a->expanded_weights, a->expanded_source_meta, a->unique_count,
+                              a->expanded_count, a->expert_prefix, a->expert_counts, a->expert_offsets, a->source_offsets,
+                              a->source_expert_prefix, a->errors, a->stats, a->transport_timestamps_ns, a->expected_receive_counts,
+                              a->channel_stats, a->channel_timestamps_ns, a->receive_expand_overlap, a->receive_prefix_state,
+                              a->prefix_tx_timestamps_ns};
+    for (const void* pointer : required)
+        if (!pointer) return set_error(PCIE_EP_E_INVALID, "an output pool pointer is NULL");
+    if (a->expanded_capacity_rows <= 0) return set_error(PCIE_EP_E_INVALID, "expanded capacity must be positive");
+
+    std::memset(&s, 0, sizeof s);
+    s.z = rt->z;
+    for (int rank = 0; rank < d.num_ranks; ++rank) s.seg[rank] = rt->segments[rank];
+    s.local_rank = rt->config.local_rank;
+    s.tx_waves = rt->tx_waves;
+    s.rx_waves = rt->rx_waves;
+    s.fuse_expand = rt->config.fuse_receive_expand ? 1 : 0;
+    s.expand = a->expand ? 1 : 0;
+    s.alignment = a->alignment;
+    s.num_tokens = a->num_tokens;
+    s.zero_padding = a->zero_padding ? 1 : 0;
+    s.reuse_plan = a->reuse_plan ? 1 : 0;
+    s.counts_ack_skip_source = rt->counts_ack_skip_source;
+    s.timeout_ticks = uint64_t(rt->config.timeout_ms) * 1000 * kTicksPerUs;
+    s.epoch = rt->epoch;
+    s.x = static_cast<const uint16_t*>(a->x);
+    s.topk_idx = a->topk_idx;
+    s.topk_weights = a->topk_weights;
+    char* plan = static_cast<char*>(a->plan);
+    s.plan_mask = reinterpret_cast<uint32_t*>(plan + rt->plan.mask);
+    s.plan_rank_ord = reinterpret_cast<int32_t*>(plan + rt->plan.rank_ord);
+    s.plan_exp_idx = reinterpret_cast<int32_t*>(plan + rt->plan.exp_idx);
+    s.plan_exp_ord = reinterpret_cast<int32_t*>(plan + rt->plan.exp_ord);
+    s.plan_counts = reinterpret_cast<int32_t*>(plan + rt->plan.counts);
+    s.plan_chan_counts = reinterpret_cast<int32_t*>(plan + rt->plan.chan_counts);
+    s.plan_chan_remote = reinterpret_cast<int32_t*>(plan + rt->plan.chan_remote);
+    s.chan_remote_tokens = rt->chan_remote_tokens;
+    s.unique_payload = static_cast<uint16_t*>(a->unique_payload);
+    s.unique_topk_idx = a->unique_topk_idx;
+    s.unique_topk_weights = a->unique_topk_weights;
+    s.unique_source_meta = a->unique_source_meta;
+    s.unique_expert_ordinals = a->unique_expert_ordinals;
+    s.expanded_payload = static_cast<uint16_t*>(a->expanded_payload);
+    s.expanded_expert_idx = a->expanded_expert_idx;
+    s.expanded_weights = a->expanded_weights;
+    s.expanded_source_meta = a->expanded_source_meta;
+    s.expanded_capacity = a->expanded_capacity_rows;
+    s.unique_count = a->unique_count;
+    s.expanded_count = a->expanded_count;
+    s.expert_prefix = a->expert_prefix;
+    s.expert_counts = a->expert_counts;
+    s.expert_offsets = a->expert_offsets;
+    s.source_offsets = a->source_offsets;
+    s.source_expert_prefix = a->source_expert_prefix;
+    s.errors = a->errors;
+    s.stats = a->stats;
+    s.transport_timestamps_ns = a->transport_timestamps_ns;
+    s.expected_receive_counts = a->expected_receive_counts;
+    s.channel_stats = a->channel_stats;
+    s.channel_timestamps_ns = a->channel_timestamps_ns;
+    s.receive_expand_overlap = a->receive_expand_overlap;
+    s.receive_prefix_state = a->receive_prefix_state;
+    s.prefix_tx_timestamps_ns = a->prefix_tx_timestamps_ns;
+    s.metadata_delay = rt->metadata_delay;
+    s.tx_delay = rt->tx_delay;
+    s.rx_delay = rt->rx_delay;
+    s.scatter_delay = rt->scatter_delay;
+    s.prefix_delay = rt->prefix_delay;
+    s.control_abort_after = rt->control_abort_after;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pcie_ep_abi_version(void) { return PCIE_EP_ABI_VERSION; }
+
+const char* pcie_ep_last_error(void) { return g_last_error.c_str(); }
+
+int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes) {
+    Dimensions dims;
+    if (int status = check_config(config, dims)) return status;
+    if (!sizes) return set_error(PCIE_EP_E_INVALID, "sizes is NULL");
+    const SegmentLayout z = make_segment_layout(dims);
+    std::memset(sizes, 0, sizeof *sizes);
+    sizes->unique_rows = unique_capacity(dims);
+    sizes->expanded_rows = expanded_capacity(dims);
+    sizes->plan_bytes = int64_t(plan_layout(dims).bytes);
+    sizes->segment_bytes = int64_t(z.size_bytes);
+    sizes->slot_stride = int64_t(z.slot_stride);
+    sizes->local_experts = z.local_experts;
+    sizes->payload_bytes = z.payload_bytes;
+    sizes->meta_bytes = z.meta_bytes;
+    sizes->mailbox_dwords = z.mailbox_dwords;
+    sizes->transport_threads = transport_threads(config->tx_waves ? config->tx_waves : kDefaultTxWaves,
+                                                 config->rx_waves ? config->rx_waves : kDefaultRxWaves);
+    return 0;
+}
+
+int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) {
+    Dimensions dims;
+    if (int status = check_config(config, dims)) return status;
+    if (!out) return set_error(PCIE_EP_E_INVALID, "runtime output pointer is NULL");
+    *out = nullptr;
+    int device_count = 0;
+    if (hipGetDeviceCount(&device_count) != hipSuccess || device_count <= config->device)
+        return set_error(PCIE_EP_E_HIP, "no HIP device %d is available: the host-staged runtime needs a GPU", config->device);
+    HIP_TRY(hipSetDevice(config->device));
+    auto rt = std::make_unique<pcie_ep_runtime>();
+    rt->config = *config;
+    rt->z = make_segment_layout(dims);
+    rt->plan = plan_layout(dims);
+    if (config->tx_waves) rt->tx_waves = config->tx_waves;
+    if (config->rx_waves) rt->rx_waves = config->rx_waves;
+
+    // Pinned, fine-grained, GPU-mapped segments (the reference registers
+    // /dev/shm mappings: advanced_shared_memory.hpp:264-288).  First touch is
+    // by this thread under the requested NUMA policy, then zeroed: a zero
+    // sequence word means "never written".
+    const bool bind = config->staging_numa_node >= 0;
+    unsigned long node_mask[16] = {};
+    if (bind) {
+        node_mask[config->staging_numa_node / 64] = 1ul << (config->staging_numa_node % 64);
+        if (syscall(SYS_set_mempolicy, MPOL_BIND, node_mask, sizeof(node_mask) * 8) != 0)
+            return set_error(PCIE_EP_E_INVALID, "set_mempolicy(MPOL_BIND, node %d) failed", config->staging_numa_node);
+    }
+    int status = 0;
+    for (int rank = 0; rank < dims.num_ranks && !status; ++rank) {
+        void* pointer = nullptr;
+        const unsigned flags = hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable | (bind ? hipHostMallocNumaUser : 0u);
+        const hipError_t allocated = hipHostMalloc(&pointer, rt->z.size_bytes, flags);
+        if (allocated != hipSuccess) {
+            status = set_error(PCIE_EP_E_HIP, "hipHostMalloc of a %zu-byte source segment failed: %s", rt->z.size_bytes, hipGetErrorString(allocated));
+            break;
+        }
+        std::memset(pointer, 0, rt->z.size_bytes);
+        rt->segments[rank] = static_cast<char*>(pointer);
+    }
+    if (bind) syscall(SYS_set_mempolicy, MPOL_DEFAULT, nullptr, 0);
+    if (!status) {
+        const size_t history = size_t(dims.channels) * ((dims.max_tokens + dims.channels - 1) / dims.channels) * 4;
+        hipError_t error = hipMalloc(reinterpret_cast<void**>(&rt->epoch), 256);
+        if (error == hipSuccess) error = hipMemset(rt->epoch, 0, 256);
+        if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->chan_remote_tokens), history);
+        if (error == hipSuccess) error = hipMemset(rt->chan_remote_tokens, 0, history);
+        if (error == hipSuccess) error = hipDeviceSynchronize();
+        if (error != hipSuccess) status = set_error(PCIE_EP_E_HIP, "device workspace allocation failed: %s", hipGetErrorString(error));
+    }
+    if (status) {
+        for (char* segment : rt->segments)
+            if (segment) (void)hipHostFree(segment);
+        if (rt->epoch) (void)hipFree(rt->epoch);
+        if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
+        return status;
+    }
+    if (config->peer_threads > 0 && dims.num_ranks > 1)
+        rt->peers = std::make_unique<PeerEmulator>(rt->z, config->local_rank, rt->segments, config->peer_threads, config->timeout_ms);
+    *out = rt.release();
+    return 0;
+}
+
+int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
+    if (!rt) return 0;
+    rt->closed = true;
+    rt->peers.reset();  // joins the emulator threads before the segments go away
+    int status = 0;
+    for (char*& segment : rt->segments) {
+        if (segment && hipHostFree(segment) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a source segment failed");
+        segment = nullptr;
+    }
+    if (rt->epoch) (void)hipFree(rt->epoch);
+    if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
+    delete rt;
+    return status;
+}
+
+int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, void* stream_handle) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    DeviceState state;
+    if (int status = build_state(rt, args, state)) return status;
+    hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+    // Kernel sequence of launch_dispatch (advanced.hpp:472-523), three launches:
+    //   prologue  = begin_epoch + route_flags + stable_ordinals + prepare_channels + publish_counts
+    //   transport = the channel kernel (TX, RX, receive prefixes, fused expand)
+    //   epilogue  = copy_local_tokens + zero_padding + reduce_statistics
+    // and the separate expand when receive/expand fusion is off.
+    HIP_TRY(launch_prologue(state, stream));
+    HIP_TRY(launch_transport(state, stream));
+    HIP_TRY(launch_epilogue(state, stream));
+    if (state.expand && !state.fuse_expand) HIP_TRY(launch_expand(state, stream));
+    return 0;
+}
+
+int pcie_ep_expand_unique(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, void* stream_handle) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    DeviceState state;
+    if (int status = build_state(rt, args, state)) return status;
+    state.expand = 1;
+    HIP_TRY(launch_expand(state, static_cast<hipStream_t>(stream_handle)));
+    return 0;
+}
+
+int pcie_ep_set_test_delays(pcie_ep_runtime* rt, uint64_t metadata_ns, uint64_t tx_ns, uint64_t rx_ns, uint64_t scatter_ns) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    rt->metadata_delay = ns_to_ticks(metadata_ns);
+    rt->tx_delay = ns_to_ticks(tx_ns);
+    rt->rx_delay = ns_to_ticks(rx_ns);
+    rt->scatter_delay = ns_to_ticks(scatter_ns);
+    return 0;
+}
+int pcie_ep_set_test_prefix_delay_ns(pcie_ep_runtime* rt, uint64_t delay_ns) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    rt->prefix_delay = ns_to_ticks(delay_ns);
+    return 0;
+}
+int pcie_ep_set_test_control_abort_after_ns(pcie_ep_runtime* rt, uint64_t delay_ns) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    rt->control_abort_after = ns_to_ticks(delay_ns);
+    return 0;
+}
+int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* rt, int32_t source) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    if (source < -1 || source >= rt->z.dims.num_ranks) return set_error(PCIE_EP_E_INVALID, "invalid test counts source");
+    rt->counts_ack_skip_source = source;
+    return 0;
+}
+
+int pcie_ep_device_numa_node(int32_t device) {
+    char bus_id[64] = {};
+    if (hipDeviceGetPCIBusId(bus_id, sizeof bus_id, device) != hipSuccess) return -1;
+    std::string bus = bus_id;
+    for (auto& character : bus) character = char(std::tolower(character));
+    std::ifstream file("/sys/bus/pci/devices/" + bus + "/numa_node");
+    int node = -1;
+    file >> node;
+    return node;
+}
+
+static uint64_t* host_signal(pcie_ep_runtime* rt, int32_t segment_rank, int32_t which, int32_t index) {
+    if (!rt || rt->closed || segment_rank < 0 || segment_rank >= rt->z.dims.num_ranks) return nullptr;
+    char* segment = rt->segments[segment_rank];
+    switch (which) {
+        case 0: return signal_at(segment, rt->z.abort_offset);
+        case 1: return index >= 0 && index < rt->z.dims.channels ? signal_at(segment, rt->z.channel_abort_offset, index) : nullptr;
+        case 2: return signal_at(segment, rt->z.counts_ready_offset);
+        case 3: return index >= 0 && index < rt->z.dims.num_ranks ? signal_at(segment, rt->z.counts_consumed_offset, index) : nullptr;
+        default: return nullptr;
+    }
+}
+
+int pcie_ep_host_signal_store(pcie_ep_runtime* rt, int32_t segment_rank, int32_t which, int32_t index, uint64_t value) {
+    uint64_t* signal = host_signal(rt, segment_rank, which, index);
+    if (!signal) return set_error(PCIE_EP_E_INVALID, "no such host signal");
+    std::atomic_ref<uint64_t>(*signal).store(value, std::memory_order_release);
+    return 0;
+}
+int pcie_ep_host_signal_load(pcie_ep_runtime* rt, int32_t segment_rank, int32_t which, int32_t index, uint64_t* value) {
+    uint64_t* signal = host_signal(rt, segment_rank, which, index);
+    if (!signal || !value) return set_error(PCIE_EP_E_INVALID, "no such host signal");
+    *value = std::atomic_ref<uint64_t>(*signal).load(std::memory_order_acquire);
+    return 0;
+}
+
+int pcie_ep_quantize_fp8(const void* x, uint8_t* codes, float* scales, int32_t tokens, int32_t hidden, void* stream) {
+    if (tokens < 0 || hidden <= 0 || (tokens && (!x || !codes || !scales))) return set_error(PCIE_EP_E_INVALID, "bad quantize arguments");
+    HIP_TRY(launch_quantize(static_cast<const uint16_t*>(x), codes, scales, tokens, hidden, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+int pcie_ep_dequantize_fp8(const uint8_t* codes, const float* scales, void* out, int32_t tokens, int32_t hidden, void* stream) {
+    if (tokens < 0 || hidden <= 0 || (tokens && (!out || !codes || !scales))) return set_error(PCIE_EP_E_INVALID, "bad dequantize arguments");
+    HIP_TRY(launch_dequantize(codes, scales, static_cast<uint16_t*>(out), tokens, hidden, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, double* h2d_gbps, double* d2h_gbps) {
+    if (bytes <= 0 || repeats < 1 || !h2d_gbps || !d2h_gbps) return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
+    HIP_TRY(hipSetDevice(device));
+    void *host = nullptr, *dev = nullptr;
+    HIP_TRY(hipHostMalloc(&host, size_t(bytes), hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable));
+    std::memset(host, 1, size_t(bytes));
+    hipStream_t stream = nullptr;
+    hipEvent_t begin = nullptr, end = nullptr;
+    hipError_t status = hipMalloc(&dev, size_t(bytes));
+    if (status == hipSuccess) status = hipStreamCreate(&stream);
+    if (status == hipSuccess) status = hipEventCreate(&begin);
+    if (status == hipSuccess) status = hipEventCreate(&end);
+    double best[2] = {0.0, 0.0};
+    for (int direction = 0; direction < 2 && status == hipSuccess; ++direction) {
+        for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+            status = hipEventRecord(begin, stream);
+            if (status == hipSuccess)
+                status = direction == 0 ? hipMemcpyAsync(dev, host, size_t(bytes), hipMemcpyHostToDevice, stream)
+                                        : hipMemcpyAsync(host, dev, size_t(bytes), hipMemcpyDeviceToHost, stream);
+            if (status == hipSuccess) status = hipEventRecord(end, stream);
+            if (status == hipSuccess) status = hipEventSynchronize(end);
+            float ms = 0.0f;
+            if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
+            if (status == hipSuccess && i > 0 && ms > 0.0f) {
+                const double rate = double(bytes) / (ms * 1e6);
+                if (rate > best[direction]) best[direction] = rate;
+            }
+        }
+    }
+    if (begin) (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    if (stream) (void)hipStreamDestroy(stream);
+    if (dev) (void)hipFree(dev);
+    (void)hipHostFree(host);
+    if (status != hipSuccess) return set_error(PCIE_EP_E_HIP, "pinned copy measurement failed: %s", hipGetErrorString(status));
+    *h2d_gbps = best[0];
+    *d2h_gbps = best[1];
+    return 0;
+}
+
+// ---- peer emulator -----------------------------------------------------------------
+
+#define NEED_PEERS(rt)                                                                                        \
+    if (!(rt) || (rt)->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");    \
+    if (!(rt)->peers) return set_error(PCIE_EP_E_STATE, "this runtime was created without a host peer emulator")
+
+int pcie_ep_peer_set_source(pcie_ep_runtime* rt, int32_t rank, const void* x, const int64_t* topk_idx, const float* weights, int32_t tokens) {
+    NEED_PEERS(rt);
+    if (tokens > 0 && (!x || !topk_idx)) return set_error(PCIE_EP_E_INVALID, "peer inputs are NULL");
+    std::string error;
+    const int status = rt->peers->set_source(rank, static_cast<const uint16_t*>(x), topk_idx, weights, tokens, error);
+    return status ? set_error(status, "%s", error.c_str()) : 0;
+}
+int pcie_ep_peers_start(pcie_ep_runtime* rt, int32_t epochs, uint32_t flags) {
+    NEED_PEERS(rt);
+    std::string error;
+    const int status = rt->peers->start(epochs, flags, error);
+    return status ? set_error(status, "%s", error.c_str()) : 0;
+}
+int pcie_ep_peers_wait_staged(pcie_ep_runtime* rt, int32_t timeout_ms) {
+    NEED_PEERS(rt);
+    std::string error;
+    const int status = rt->peers->wait_staged(timeout_ms, error);
+    return status ? set_error(status, "%s", error.c_str()) : 0;
+}
+int pcie_ep_peers_wait(pcie_ep_runtime* rt, int32_t timeout_ms) {
+    NEED_PEERS(rt);
+    std::string error;
+    const int status = rt->peers->wait(timeout_ms, error);
+    return status ? set_error(status, "%s", error.c_str()) : 0;
+}
+int pcie_ep_peers_cancel(pcie_ep_runtime* rt) {
+    NEED_PEERS(rt);
+    rt->peers->cancel();
+    return 0;
+}
+int pcie_ep_peer_captured_count(pcie_ep_runtime* rt, int32_t rank, int64_t* count) {
+    NEED_PEERS(rt);
+    const int64_t value = rt->peers->captured_count(rank);
+    if (value < 0 || !count) return set_error(PCIE_EP_E_INVALID, "no such peer rank");
+    *count = value;
+    return 0;
+}
+int pcie_ep_peer_captured_copy(pcie_ep_runtime* rt, int32_t rank, int32_t* tokens, int32_t* rank_ordinals, uint8_t* payload, float* scales,
+                               int32_t* expert_idx, int32_t* expert_ordinals, float* weights, uint32_t* destination_masks) {
+    NEED_PEERS(rt);
+    if (rt->peers->captured_copy(rank, tokens, rank_ordinals, payload, scales, expert_idx, expert_ordinals, weights, destination_masks))
+        return set_error(PCIE_EP_E_INVALID, "no such peer rank");
+    return 0;
+}
+int pcie_ep_peers_inject_fault(pcie_ep_runtime* rt, int32_t rank, int32_t fault) {
+    NEED_PEERS(rt);
+    if (rt->peers->inject_fault(rank, fault)) return set_error(PCIE_EP_E_INVALID, "no such peer rank or fault");
+    return 0;
+}
+
+// ---- host implementations shared with the emulator -----------------------------------
+
+int pcie_ep_host_quantize_fp8(const void* x, uint8_t* codes, float* scales, int32_t tokens, int32_t hidden) {
+    if (tokens < 0 || hidden < 0 || (tokens && hidden && (!x || !codes)) || (tokens && !scales)) return set_error(PCIE_EP_E_INVALID, "bad quantize arguments");
+    host_quantize_fp8(static_cast<const uint16_t*>(x), codes, scales, tokens, hidden);
+    return 0;
+}
+int pcie_ep_host_dequantize_fp8(const uint8_t* codes, const float* scales, void* out, int32_t tokens, int32_t hidden) {
+    if (tokens < 0 || hidden < 0 || (tokens && hidden && (!out || !codes)) || (tokens && !scales)) return set_error(PCIE_EP_E_INVALID, "bad dequantize arguments");
+    host_dequantize_fp8(codes, scales, static_cast<uint16_t*>(out), tokens, hidden);
+    return 0;
+}
+int pcie_ep_host_source_layout(const int64_t* topk_idx, int32_t tokens, int32_t topk, int32_t num_ranks, int32_t num_experts, uint32_t* mask,
+                               int32_t* rank_ordinals, int32_t* expert_indices, int32_t* expert_ordinals, int32_t* counts) {
+    if (tokens < 0 || topk < 1 || topk > kMaxTopk || num_ranks < 1 || num_ranks > kMaxRanks || num_experts < num_ranks ||
+        num_experts % num_ranks || !counts || (tokens && (!topk_idx || !mask || !rank_ordinals || !expert_indices || !expert_ordinals)))
+        return set_error(PCIE_EP_E_INVALID, "bad layout arguments");
+    return host_source_layout(topk_idx, tokens, topk, num_ranks, num_experts, mask, rank_ordinals, expert_indices, expert_ordinals, counts);
+}
+
+}  // extern "C"

@@ -1,0 +1,809 @@
+// Channel transport kernel: one workgroup per channel, wavefronts specialised
+// into TX control (+ guardian), RX control (+ receive prefixes), TX payload
+// workers and RX/scatter workers.
+//
+// Replaces advanced_transport_pipelined and its roles
+// (csrc/kernels/host_staged/fused_receive.cuh:333-360;
+// advanced_dispatch.cuh:287-477 tx_control, :479-625 rx_control, :627-689
+// tx_worker; fused_receive.cuh:199-305 producer/consumer) and, for the unique
+// layout, advanced_transport (advanced_dispatch.cuh:919-958).
+//
+// Differences that come from designing for 64-lane wavefronts:
+//  * A payload worker is ONE wavefront that owns a whole row: 14 x 16-byte
+//    loads per lane are issued back to back (896 vectors of a 14 336-byte BF16
+//    row), the row lives in registers, and the same wavefront stores it to
+//    every destination expert row.  The staged row is read once, there is no
+//    LDS tile and no producer/consumer hand-off (the reference stages through
+//    shared memory with 3+3 warps per ticket).
+//  * Control wavefronts work on 64 candidates at a time with ballots: TX control
+//    derives ring slots and per-destination descriptor ordinals for 64 tokens
+//    from popcounts of ballots; RX control probes up to 64/P descriptors per
+//    source per iteration instead of one source per iteration.
+//  * Workers publish their own descriptors and payload ACKs as soon as their
+//    own fence has completed; control wavefronts only reserve and hand out work.
+#include "device_common.h"
+#include "launch.h"
+#include "row_codec.h"
+
+namespace pcie_ep {
+
+namespace {
+
+constexpr int kTxRing = 32;
+constexpr int kRxRing = 32;
+constexpr int kScratchDwords = 128;  // per worker wavefront: one slot metadata record
+
+struct TxTicket {
+    int token;
+    int ordinal;  // position among this channel's remote tokens
+    uint32_t endpoints;
+    int pad;
+    int descriptor_ordinal[kMaxRanks];
+};
+
+struct RxTicket {
+    int source;
+    int slot;
+    int token;
+    int descriptor_ordinal;
+    uint64_t payload_sequence;
+};
+
+struct Queues {
+    int abort;
+    int tx_finished;
+    int rx_finished;
+    int tx_head;   // tickets published by TX control
+    int tx_total;  // -1 until every ticket is published
+    int rx_head;
+    int rx_total;
+    int pad;
+    int tx_done[kMaxTxWaves];  // tickets completed by each TX worker
+    int rx_done[kMaxRxWaves];
+    TxTicket tx[kTxRing];
+    RxTicket rx[kRxRing];
+    uint32_t scratch[kMaxTxWaves + kMaxRxWaves][kScratchDwords];
+};
+
+__device__ __forceinline__ bool ticket_slot_free(const int* done, int workers, int ring, int ticket) {
+    const int previous = ticket - ring;
+    if (previous < 0) return true;
+    return lds_load(done + previous % workers) > previous / workers;
+}
+
+// Wait until ticket `ticket` is published.  Returns 1 when available, -1 to exit.
+__device__ inline int wait_ticket(Queues& q, const int* head, const int* total, int ticket, int lane) {
+    while (true) {
+        int action = 0;
+        if (lane == 0) {
+            if (lds_load(&q.abort)) action = -1;
+            else if (lds_load(head) > ticket) action = 1;
+            else {
+                const int limit = lds_load(total);
+                if (limit >= 0 && ticket >= limit) action = -1;
+            }
+        }
+        action = broadcast_first(action);
+        if (action) return action;
+        backoff();
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Receive prefixes (advanced_layout.cuh:94-195).  One wavefront of the grid is
+// elected by a device-scope CAS; it waits for every source's counts_ready,
+// folds the mailboxes in rank order and publishes a generation-valued READY.
+// ---------------------------------------------------------------------------------------
+__device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks, local = z.local_experts, channels = z.dims.channels;
+    const int me = state.local_rank;
+    const uint64_t epoch = *state.epoch;
+    const uint64_t start = now_ticks();
+    HealthCheck health(state, start);
+    if (lane == 0) {
+        state.prefix_tx_timestamps_ns[0] = ticks_to_ns(start);
+        test_delay(state.prefix_delay);
+    }
+    // All sources are polled in parallel, one lane each.
+    bool ready = lane >= ranks;
+    while (true) {
+        if (!ready) ready = load_acquire_system(signal_at(state.seg[lane], z.counts_ready_offset)) == epoch;
+        if (__all(ready)) break;
+        if (health.poll(state, lane)) {
+            if (lane == 0) record_error(state, kErrCountsReadyWait);
+            return false;
+        }
+        backoff();
+    }
+    fence_acquire_system();
+    // Per-source unique counts -> source_offsets (lane = source).
+    int unique = 0;
+    if (lane < ranks) unique = mailbox_at(z, state.seg[lane], me)[0];
+    int inclusive = unique;
+    for (int offset = 1; offset < kMaxRanks; offset <<= 1) {
+        const int other = __shfl_up(inclusive, offset);
+        if (lane >= offset) inclusive += other;
+    }
+    if (lane < ranks) state.source_offsets[lane + 1] = inclusive;
+    if (lane == 0) state.source_offsets[0] = 0;
+    const int total_unique = __shfl(inclusive, ranks - 1);
+    // Expert branches: lane = local expert; all sources' loads are issued first.
+    int carry_offset = 0;
+    int64_t expanded_total = 0;
+    for (int begin = 0; begin < local; begin += kWave) {
+        const int expert = begin + lane;
+        int counts[kMaxRanks];
+#pragma unroll
+        for (int source = 0; source < kMaxRanks; ++source)
+            counts[source] = (source < ranks && expert < local) ? mailbox_at(z, state.seg[source], me)[1 + expert] : 0;
+        int running = 0;
+#pragma unroll
+        for (int source = 0; source < kMaxRanks; ++source) {
+            if (source < ranks && expert < local) state.source_expert_prefix[source * local + expert] = running;
+            running += counts[source];
+        }
+        const int padded = (running + state.alignment - 1) / state.alignment * state.alignment;
+        int scan = padded;
+        for (int offset = 1; offset < kWave; offset <<= 1) {
+            const int other = __shfl_up(scan, offset);
+            if (lane >= offset) scan += other;
+        }
+        const int exclusive = carry_offset + scan - padded;
+        if (expert < local) {
+            state.expert_counts[expert] = running;
+            state.expert_offsets[expert] = exclusive;
+            state.expert_prefix[expert] = exclusive + running;
+            if (expert == local - 1) state.expert_offsets[local] = exclusive + padded;
+        }
+        carry_offset += __shfl(scan, kWave - 1);
+        int sum = running;
+        for (int offset = 32; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset);
+        expanded_total += sum;
+    }
+    // Expected tokens per (channel, source) for this receiver.
+    for (int index = lane; index < channels * ranks; index += kWave) {
+        const int channel = index / ranks, source = index % ranks;
+        state.expected_receive_counts[index] = mailbox_at(z, state.seg[source], me)[1 + local + channel];
+    }
+    if (lane == 0) {
+        *state.unique_count = total_unique;
+        *state.expanded_count = expanded_total;
+    }
+    // ACK a source only after every lane captured its counts: the source may
+    // overwrite the mailbox for the next epoch afterwards (advanced_layout.cuh:91-93).
+    __threadfence_system();
+    if (lane < ranks && lane != me && lane != state.counts_ack_skip_source)
+        store_release_system(signal_at(state.seg[lane], z.counts_consumed_offset, me), epoch);
+    return true;
+}
+
+__device__ bool prepare_receive_prefixes(const DeviceState& state, int lane) {
+    const uint64_t epoch = *state.epoch;
+    int claimed = 0;
+    if (lane == 0) {
+        unsigned long long expected = 0;
+        claimed = atomicCAS(reinterpret_cast<unsigned long long*>(state.receive_prefix_state), expected, epoch) == 0ull;
+    }
+    if (broadcast_first(claimed)) {
+        const bool success = compute_receive_prefixes(state, lane);
+        __threadfence();
+        if (lane == 0) {
+            state.prefix_tx_timestamps_ns[1] = ticks_to_ns(now_ticks());
+            store_release_device(state.receive_prefix_state + 1, success ? epoch : kPrefixFailed);
+        }
+    }
+    int success = 0;
+    if (lane == 0) {
+        while (true) {
+            const uint64_t value = load_acquire_device(state.receive_prefix_state + 1);
+            if (value == epoch) { success = 1; break; }
+            // The elected producer owns the timeout; waiters only read device flags.
+            if (value == kPrefixFailed || load_error_code(state)) break;
+            backoff();
+        }
+    }
+    success = broadcast_first(success);
+    __threadfence();
+    return success != 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// TX control + guardian
+// ---------------------------------------------------------------------------------------
+__device__ void tx_control(const DeviceState& state, Queues& q, int channel, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks, channels = z.dims.channels, me = state.local_rank;
+    const int slots = z.dims.payload_slots;
+    const int stride = (z.dims.max_tokens + channels - 1) / channels;
+    char* own = state.seg[me];
+    const uint64_t epoch = *state.epoch;
+    const uint64_t start = now_ticks();
+    HealthCheck health(state, start);
+    if (lane == 0) state.channel_timestamps_ns[channel * 2] = ticks_to_ns(start);
+    const int tokens = state.num_tokens;
+    const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;
+    const uint64_t below = lanes_below(lane);
+    int produced = 0;
+    int reserved[kMaxRanks];
+#pragma unroll
+    for (int rank = 0; rank < kMaxRanks; ++rank) reserved[rank] = 0;
+    bool failed = false;
+    int64_t stage_busy = 0;
+
+    for (int base = 0; base < candidates && !failed; base += kWave) {
+        const int candidate = base + lane;
+        const int token = channel + candidate * channels;
+        const uint32_t remote = candidate < candidates ? (state.plan_mask[token] & ~(1u << me)) : 0u;
+        const uint64_t batch = __ballot(remote != 0);
+        if (!batch) continue;
+        const int ordinal = produced + __popcll(batch & below);
+        int my_descriptor[kMaxRanks];
+#pragma unroll
+        for (int rank = 0; rank < kMaxRanks; ++rank) {
+            my_descriptor[rank] = 0;
+            if (rank < ranks) {
+                const uint64_t hits = __ballot((remote >> rank) & 1u);
+                my_descriptor[rank] = reserved[rank] + __popcll(hits & below);
+                reserved[rank] += __popcll(hits);
+            }
+        }
+        // Ring history: which token occupied ordinal i (needed when a slot is reused).
+        if (remote) state.chan_remote_tokens[size_t(channel) * stride + ordinal] = token;
+        bool pending = remote != 0;
+        while (true) {
+            if (pending && ticket_slot_free(q.tx_done, state.tx_waves, kTxRing, ordinal)) {
+                TxTicket& ticket = q.tx[ordinal % kTxRing];
+                ticket.token = token;
+                ticket.ordinal = ordinal;
+                ticket.endpoints = remote;
+#pragma unroll
+                for (int rank = 0; rank < kMaxRanks; ++rank)
+                    if (rank < ranks) ticket.descriptor_ordinal[rank] = my_descriptor[rank];
+                pending = false;
+            }
+            const uint64_t still = __ballot(pending);
+            const int first_pending = still ? __builtin_ctzll(still) : kWave;
+            const int head = produced + __popcll(batch & lanes_below(first_pending));
+            __threadfence();  // ring history + ticket bodies before the head
+            fence_workgroup();
+            if (lane == 0) lds_store(&q.tx_head, head);
+            if (!still) break;
+            ++stage_busy;
+            if (health.poll(state, lane) || broadcast_first(lds_load(&q.abort))) {
+                failed = true;
+                break;
+            }
+            backoff();
+        }
+        produced += __popcll(batch);
+    }
+    if (lane == 0) lds_store(&q.tx_total, produced);
+
+    // Wait for the workers, then drain the ACKs of the last ring window: earlier
+    // slots were checked when they were reused (advanced_dispatch.cuh:229-285).
+    // Lanes poll different (ordinal, destination) pairs in parallel.
+    bool drained = failed;
+    int drain_ordinal = produced > slots ? produced - slots : 0;
+    bool workers_finished = false;
+    while (true) {
+        int verdict = 0;
+        if (lane == 0) {
+            if (lds_load(&q.abort)) verdict = -1;
+        }
+        verdict = broadcast_first(verdict);
+        if (verdict < 0) break;
+        if (!workers_finished) {
+            int done = lane < state.tx_waves ? lds_load(q.tx_done + lane) : 0;
+            for (int offset = 32; offset > 0; offset >>= 1) done += __shfl_xor(done, offset);
+            workers_finished = done >= produced;
+        }
+        if (workers_finished && !drained) {
+            // Each pass checks up to 64 / P ordinals with one lane per destination.
+            const int per_pass = kWave / ranks;
+            const int my_ordinal = drain_ordinal + lane / ranks;
+            const int destination = lane % ranks;
+            bool acked = true;
+            if (lane < per_pass * ranks && my_ordinal < produced) {
+                const int token = state.chan_remote_tokens[size_t(channel) * stride + my_ordinal];
+                const uint32_t remote = state.plan_mask[token] & ~(1u << me);
+                if ((remote >> destination) & 1u)
+                    acked = load_acquire_system(ack_at(z, own, channel, my_ordinal % slots, destination)) == sequence(epoch, token);
+            }
+            const uint64_t missing = __ballot(!acked);
+            if (!missing) drain_ordinal += per_pass;
+            else drain_ordinal += __builtin_ctzll(missing) / ranks;  // everything before the first miss is done
+            if (drain_ordinal >= produced) drained = true;
+        }
+        if (workers_finished && drained) {
+            if (lane == 0 && !lds_load(&q.tx_finished)) lds_store(&q.tx_finished, 1);
+            if (broadcast_first(lds_load(&q.rx_finished))) break;
+        }
+        // Guardian: this wavefront outlives TX so that a stalled RX still times out.
+        const bool unhealthy = health.poll(state, lane);
+        const bool forced = channel == 0 && state.control_abort_after && now_ticks() - start >= state.control_abort_after;
+        if (unhealthy || broadcast_first(forced ? 1 : 0)) {
+            if (lane == 0) {
+                record_error(state, kErrRingProgressWait);
+                lds_store(&q.abort, 1);
+            }
+            break;
+        }
+        backoff();
+    }
+    if (lane == 0) {
+        lds_store(&q.tx_finished, 1);
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatTxStageBusy),
+                  static_cast<unsigned long long>(stage_busy));
+        // Only this wavefront writes the channel's mapped abort word.
+        if (lds_load(&q.abort)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// RX control
+// ---------------------------------------------------------------------------------------
+__device__ void rx_control(const DeviceState& state, Queues& q, int channel, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks, me = state.local_rank;
+    if (!prepare_receive_prefixes(state, lane)) {
+        if (lane == 0) {
+            lds_store(&q.abort, 1);
+            lds_store(&q.rx_total, 0);
+            lds_store(&q.rx_finished, 1);
+        }
+        return;
+    }
+    const uint64_t epoch = *state.epoch;
+    const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
+    const int source = lane / lookahead, ahead = lane % lookahead;
+    const bool member = source < ranks && source != me;
+    const int expected = member ? state.expected_receive_counts[channel * ranks + source] : 0;
+    int total = ahead == 0 ? expected : 0;
+    for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
+    if (lane == 0) lds_store(&q.rx_total, total);
+    const uint64_t below = lanes_below(lane);
+    const uint64_t group_mask = lookahead >= 64 ? ~0ull : ((1ull << lookahead) - 1ull);
+    int consumed = 0, issued = 0;
+    int64_t not_ready = 0;
+    bool failed = false;
+    while (issued < total && !failed) {
+        if (broadcast_first(lds_load(&q.abort))) break;
+        const int ordinal = consumed + ahead;
+        const bool want = member && ordinal < expected;
+        Descriptor* descriptor = descriptor_at(z, state.seg[member ? source : me], channel, me, want ? ordinal : 0);
+        bool ready = false;
+        if (want) ready = load_acquire_system(&descriptor->ready) == sequence(epoch, ordinal);
+        const uint64_t ready_lanes = __ballot(ready);
+        // Descriptors of one source are consumed in order: accept the leading run.
+        const uint64_t group = (ready_lanes >> (source < ranks ? source * lookahead : 0)) & group_mask;
+        const int run = __builtin_ctzll(~group | (1ull << lookahead));
+        const bool accept = ready && ahead < run;
+        const uint64_t accepted = __ballot(accept);
+        if (!accepted) {
+            ++not_ready;
+            backoff();
+            continue;
+        }
+        const int ticket_index = issued + __popcll(accepted & below);
+        int slot = 0, token = 0;
+        uint64_t payload_sequence = 0;
+        if (accept) {
+            slot = descriptor->payload_slot;
+            token = descriptor->token_index;
+            payload_sequence = descriptor->payload_sequence;
+        }
+        bool pending = accept;
+        while (true) {
+            if (pending && ticket_slot_free(q.rx_done, state.rx_waves, kRxRing, ticket_index)) {
+                RxTicket& ticket = q.rx[ticket_index % kRxRing];
+                ticket.source = source;
+                ticket.slot = slot;
+                ticket.token = token;
+                ticket.descriptor_ordinal = ordinal;
+                ticket.payload_sequence = payload_sequence;
+                // The descriptor is captured: return its credit.  The payload ACK
+                // and the local ticket slot are separate resources.
+                store_release_system(&descriptor->consumed, sequence(epoch, ordinal));
+                pending = false;
+            }
+            const uint64_t still = __ballot(pending);
+            const int first_pending = still ? __builtin_ctzll(still) : kWave;
+            const int head = issued + __popcll(accepted & lanes_below(first_pending));
+            fence_workgroup();
+            if (lane == 0) lds_store(&q.rx_head, head);
+            if (!still) break;
+            if (broadcast_first(lds_load(&q.abort))) {
+                failed = true;
+                break;
+            }
+            backoff();
+        }
+        issued += __popcll(accepted);
+        if (member) consumed += run;
+    }
+    // RX is finished when every worker has retired its tickets.
+    while (true) {
+        if (broadcast_first(lds_load(&q.abort))) break;
+        int done = lane < state.rx_waves ? lds_load(q.rx_done + lane) : 0;
+        for (int offset = 32; offset > 0; offset >>= 1) done += __shfl_xor(done, offset);
+        if (done >= issued && issued >= total) break;
+        backoff();
+    }
+    if (lane == 0) {
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxNotReady),
+                  static_cast<unsigned long long>(not_ready));
+        lds_store(&q.rx_finished, 1);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// TX payload worker
+// ---------------------------------------------------------------------------------------
+template <bool kFp8, bool kVector>
+__device__ void tx_copy_row(const DeviceState& state, const uint16_t* input, char* slot, uint32_t* scratch, int lane) {
+    const int hidden = state.z.dims.hidden;
+    float scale = 1.0f;
+    if constexpr (kFp8) scale = quantize_row<kVector>(input, reinterpret_cast<uint8_t*>(slot), hidden, lane);
+    else copy_row<kVector, false>(input, reinterpret_cast<uint16_t*>(slot), hidden, lane);
+    if (lane == 0) scratch[2] = float_bits(scale);
+}
+
+template <bool kFp8, bool kVector>
+__device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int worker, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
+    const int slots = z.dims.payload_slots, descriptors = z.dims.descriptor_slots;
+    const int stride = (z.dims.max_tokens + z.dims.channels - 1) / z.dims.channels;
+    char* own = state.seg[me];
+    const uint64_t epoch = *state.epoch;
+    uint32_t* scratch = q.scratch[worker];
+    const int meta_dwords = z.meta_bytes / 4;
+    int64_t writes = 0, deliveries = 0, credit_miss = 0;
+    for (int ticket_index = worker;; ticket_index += state.tx_waves) {
+        if (wait_ticket(q, &q.tx_head, &q.tx_total, ticket_index, lane) < 0) break;
+        fence_workgroup();
+        __threadfence();
+        const TxTicket& ticket = q.tx[ticket_index % kTxRing];
+        const int token = ticket.token, ordinal = ticket.ordinal;
+        const uint32_t endpoints = ticket.endpoints;
+        const int slot = ordinal % slots;
+        const int my_descriptor = lane < ranks ? ticket.descriptor_ordinal[lane] : 0;
+        const bool targeted = lane < ranks && ((endpoints >> lane) & 1u);
+        if (ticket_index == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(now_ticks());
+
+        // Flow control: the slot's previous occupant must be ACKed by all its
+        // targets and a descriptor entry must have been consumed before reuse
+        // (advanced_dispatch.cuh:158-187).  One lane per destination.
+        bool slot_ok = true, credit_ok = true;
+        uint64_t previous_sequence = 0;
+        if (ordinal >= slots) {
+            const int previous_token = state.chan_remote_tokens[size_t(channel) * stride + ordinal - slots];
+            const uint32_t previous_remote = state.plan_mask[previous_token] & ~(1u << me);
+            slot_ok = !(lane < ranks && ((previous_remote >> lane) & 1u));
+            previous_sequence = sequence(epoch, previous_token);
+        }
+        if (targeted && my_descriptor >= descriptors) credit_ok = false;
+        bool aborted = false;
+        while (true) {
+            if (!slot_ok) slot_ok = load_acquire_system(ack_at(z, own, channel, slot, lane)) == previous_sequence;
+            if (!credit_ok)
+                credit_ok = load_acquire_system(&descriptor_at(z, own, channel, lane, my_descriptor)->consumed) ==
+                            sequence(epoch, my_descriptor - descriptors);
+            if (__all(slot_ok && credit_ok)) break;
+            ++credit_miss;
+            if (broadcast_first(lds_load(&q.abort))) {
+                aborted = true;
+                break;
+            }
+            backoff();
+        }
+        if (aborted) break;
+        fence_acquire_system();
+
+        // Slot metadata: composed in this wavefront's LDS scratch, then copied out
+        // as consecutive dwords.  Weights are the live ones of this dispatch.
+        char* slot_base = slot_at(z, own, channel, slot);
+        for (int index = lane; index < meta_dwords; index += kWave) scratch[index] = 0;
+        fence_workgroup();
+        if (lane == 0) {
+            scratch[0] = uint32_t(token);
+            scratch[1] = state.plan_mask[token];
+        }
+        if (lane < ranks) scratch[kMetaRankOrdinalsOffset / 4 + lane] = uint32_t(state.plan_rank_ord[size_t(token) * ranks + lane]);
+        if (lane < topk) {
+            scratch[kMetaBranchOffset / 4 + lane] = uint32_t(state.plan_exp_idx[size_t(token) * topk + lane]);
+            scratch[kMetaBranchOffset / 4 + topk + lane] = uint32_t(state.plan_exp_ord[size_t(token) * topk + lane]);
+            scratch[kMetaBranchOffset / 4 + 2 * topk + lane] =
+                float_bits(state.topk_weights ? state.topk_weights[size_t(token) * topk + lane] : 1.0f);
+        }
+        if (lane == kWave - 1) test_delay(state.tx_delay);
+        tx_copy_row<kFp8, kVector>(state, state.x + size_t(token) * z.dims.hidden, slot_base, scratch, lane);
+        fence_workgroup();
+        if (lane == meta_dwords - 1 || (lane == kWave - 1 && meta_dwords > kWave)) test_delay(state.metadata_delay);
+        uint32_t* meta = reinterpret_cast<uint32_t*>(slot_base + z.meta_offset);
+        for (int index = lane; index < meta_dwords; index += kWave) meta[index] = scratch[index];
+        // Every lane's payload and metadata stores are complete at system scope
+        // before any lane publishes a descriptor.
+        __threadfence_system();
+        if (targeted) {
+            Descriptor* descriptor = descriptor_at(z, own, channel, lane, my_descriptor);
+            descriptor->payload_sequence = sequence(epoch, token);
+            descriptor->payload_slot = slot;
+            descriptor->token_index = token;
+            descriptor->rank_ordinal = int32_t(scratch[kMetaRankOrdinalsOffset / 4 + lane]);
+            store_release_system(&descriptor->ready, sequence(epoch, my_descriptor));
+        }
+        if (ticket_index == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
+        ++writes;
+        deliveries += __popc(endpoints);
+        fence_workgroup();
+        if (lane == 0) lds_store(q.tx_done + worker, ticket_index / state.tx_waves + 1);
+    }
+    if (lane == 0) {
+        auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields);
+        atomicAdd(stats + kStatHostWrites, static_cast<unsigned long long>(writes));
+        atomicAdd(stats + kStatDeliveries, static_cast<unsigned long long>(deliveries));
+        atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(deliveries));
+        atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(credit_miss));
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// RX + scatter worker
+// ---------------------------------------------------------------------------------------
+struct Destinations {
+    int count;
+    int64_t row[kMaxTopk];
+};
+
+template <bool kFp8, bool kVector>
+__device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int worker, int lane) {
+    const SegmentLayout& z = state.z;
+    const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
+    const int hidden = z.dims.hidden;
+    const uint64_t epoch = *state.epoch;
+    uint32_t* scratch = q.scratch[kMaxTxWaves + worker];
+    const int meta_dwords = z.meta_bytes / 4;
+    const bool scatter = state.expand && state.fuse_expand;
+    int64_t reads = 0;
+    for (int ticket_index = worker;; ticket_index += state.rx_waves) {
+        if (wait_ticket(q, &q.rx_head, &q.rx_total, ticket_index, lane) < 0) break;
+        fence_workgroup();
+        fence_acquire_system();
+        const RxTicket ticket = q.rx[ticket_index % kRxRing];
+        const int source = ticket.source;
+        const char* slot_base = slot_at(z, state.seg[source], channel, ticket.slot);
+        if (lane == kWave - 1) test_delay(state.rx_delay);
+
+        // Metadata first (it arrives first), payload right behind it.
+        const uint32_t* meta = reinterpret_cast<const uint32_t*>(slot_base + z.meta_offset);
+        uint32_t meta_lo = 0, meta_hi = 0;
+        if (lane < meta_dwords) meta_lo = __builtin_nontemporal_load(meta + lane);
+        if (kWave + lane < meta_dwords) meta_hi = __builtin_nontemporal_load(meta + kWave + lane);
+
+        RowVectors row;
+        const int wire_vectors = kFp8 ? hidden / 16 : hidden / 8;
+        const int wire_per_pass = kFp8 ? (kPassItems / 2) * kWave : kPassItems * kWave;
+        if constexpr (kVector) {
+            // First (usually only) pass of the row.
+            if constexpr (kFp8) {
+#pragma unroll
+                for (int j = 0; j < kPassItems / 2; ++j) {
+                    const int index = j * kWave + lane;
+                    row.v[j] = index < wire_vectors ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(slot_base) + index) : u32x4{0u, 0u, 0u, 0u};
+                }
+            } else {
+                row_load_vectors<true>(row, reinterpret_cast<const u32x4*>(slot_base), 0, wire_vectors, lane);
+            }
+        }
+        scratch[lane] = meta_lo;
+        if (kWave + lane < kScratchDwords) scratch[kWave + lane] = meta_hi;
+        fence_workgroup();
+        const int token = int(scratch[0]);
+        const float scale = bits_float(scratch[2]);
+        bool bad = token != ticket.token || ticket.payload_sequence != sequence(epoch, token);
+        if (bad) {
+            // Terminal: never forge an ACK for a slot whose identity is unknown
+            // (advanced_dispatch.cuh:607-610).
+            if (lane == 0) {
+                record_error(state, kErrPayloadSequence);
+                lds_store(&q.abort, 1);
+            }
+            break;
+        }
+
+        // Destination rows, one lane per branch.
+        int64_t my_row = -1;
+        int my_expert = -1;
+        if (scatter) {
+            if (lane < topk) {
+                const int expert = int(scratch[kMetaBranchOffset / 4 + lane]) - me * local;
+                if (int(scratch[kMetaBranchOffset / 4 + lane]) >= 0 && expert >= 0 && expert < local) {
+                    my_expert = expert;
+                    my_row = int64_t(state.expert_offsets[expert]) + state.source_expert_prefix[source * local + expert] +
+                             int(scratch[kMetaBranchOffset / 4 + topk + lane]);
+                }
+            }
+        } else if (lane == 0) {
+            my_row = int64_t(state.source_offsets[source]) + int(scratch[kMetaRankOrdinalsOffset / 4 + me]);
+        }
+        const int64_t capacity = scatter ? state.expanded_capacity : unique_capacity(z.dims);
+        if (__any(my_row >= capacity)) {
+            if (lane == 0) {
+                record_error(state, kErrExpandedCapacity);
+                lds_store(&q.abort, 1);
+            }
+            break;
+        }
+        const uint64_t destinations = __ballot(my_row >= 0);
+        uint16_t* output_base = scatter ? state.expanded_payload : state.unique_payload;
+        if (lane == kWave - 1) test_delay(state.scatter_delay);
+
+        if constexpr (kVector) {
+            const int out_vectors = hidden / 8;
+            for (int first_wire = 0; first_wire < wire_vectors; first_wire += wire_per_pass) {
+                if (first_wire > 0) {
+                    if constexpr (kFp8) {
+#pragma unroll
+                        for (int j = 0; j < kPassItems / 2; ++j) {
+                            const int index = first_wire + j * kWave + lane;
+                            row.v[j] = index < wire_vectors ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(slot_base) + index) : u32x4{0u, 0u, 0u, 0u};
+                        }
+                    } else {
+                        row_load_vectors<true>(row, reinterpret_cast<const u32x4*>(slot_base), first_wire, wire_vectors, lane);
+                    }
+                }
+                const bool last_pass = first_wire + wire_per_pass >= wire_vectors;
+                if (last_pass) {
+                    // All loads of the staged row have returned: release the host
+                    // slot.  The release orders them before the ACK store.
+                    if (lane == 0) store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                }
+                if constexpr (kFp8) {
+                    // 16 codes -> 16 BF16 (two 16-byte vectors); expanded in place from the top.
+#pragma unroll
+                    for (int j = kPassItems / 2 - 1; j >= 0; --j) {
+                        u32x4 lo, hi;
+                        dequantize_vector(row.v[j], scale, lo, hi);
+                        row.v[2 * j] = lo;
+                        row.v[2 * j + 1] = hi;
+                    }
+                }
+                uint64_t remaining = destinations;
+                while (remaining) {
+                    const int branch = __builtin_ctzll(remaining);
+                    remaining &= remaining - 1;
+                    const int64_t out_row = __shfl(my_row, branch);
+                    u32x4* output = reinterpret_cast<u32x4*>(output_base + size_t(out_row) * hidden);
+                    if constexpr (kFp8) {
+                        // Lane's wire vector j*64+lane holds elements [16*i, 16*i+16) -> output vectors 2*i, 2*i+1.
+#pragma unroll
+                        for (int j = 0; j < kPassItems / 2; ++j) {
+                            const int index = first_wire + j * kWave + lane;
+                            if (index < wire_vectors) {
+                                __builtin_nontemporal_store(row.v[2 * j], output + 2 * index);
+                                __builtin_nontemporal_store(row.v[2 * j + 1], output + 2 * index + 1);
+                            }
+                        }
+                    } else {
+                        row_store_vectors<true>(row, output, first_wire, out_vectors, lane);
+                    }
+                }
+            }
+        } else {
+            // Scalar fall-back (row length not a multiple of 16 bytes): 2-byte items.
+            for (int first = 0; first < hidden; first += kPassScalars * kWave) {
+                RowScalars items;
+#pragma unroll
+                for (int j = 0; j < kPassScalars; ++j) {
+                    const int index = first + j * kWave + lane;
+                    if (index < hidden) {
+                        if constexpr (kFp8) items.v[j] = fp8_dequantize_element(reinterpret_cast<const uint8_t*>(slot_base)[index], scale);
+                        else items.v[j] = reinterpret_cast<const uint16_t*>(slot_base)[index];
+                    }
+                }
+                if (first + kPassScalars * kWave >= hidden) {
+                    if (lane == 0) store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                }
+                uint64_t remaining = destinations;
+                while (remaining) {
+                    const int branch = __builtin_ctzll(remaining);
+                    remaining &= remaining - 1;
+                    const int64_t out_row = __shfl(my_row, branch);
+                    uint16_t* output = output_base + size_t(out_row) * hidden;
+#pragma unroll
+                    for (int j = 0; j < kPassScalars; ++j) {
+                        const int index = first + j * kWave + lane;
+                        if (index < hidden) output[index] = items.v[j];
+                    }
+                }
+            }
+            if (hidden == 0 && lane == 0)
+                store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+        }
+
+        // Row metadata (advanced_layout.cuh:207-215; layout.cuh:31-48).
+        if (scatter) {
+            if (my_row >= 0) {
+                state.expanded_expert_idx[my_row] = my_expert;
+                state.expanded_weights[my_row] = bits_float(scratch[kMetaBranchOffset / 4 + 2 * topk + lane]);
+                state.expanded_source_meta[my_row * 3] = source;
+                state.expanded_source_meta[my_row * 3 + 1] = token;
+                state.expanded_source_meta[my_row * 3 + 2] = lane;
+            }
+        } else {
+            const int64_t out_row = __shfl(my_row, 0);
+            if (lane < topk) {
+                const int expert = int(scratch[kMetaBranchOffset / 4 + lane]);
+                const bool is_local = expert >= me * local && expert < (me + 1) * local;
+                state.unique_topk_idx[out_row * topk + lane] = is_local ? expert - me * local : -1;
+                state.unique_topk_weights[out_row * topk + lane] = is_local ? bits_float(scratch[kMetaBranchOffset / 4 + 2 * topk + lane]) : 0.0f;
+                state.unique_expert_ordinals[out_row * topk + lane] = int(scratch[kMetaBranchOffset / 4 + topk + lane]);
+            }
+            if (lane == 0) {
+                state.unique_source_meta[out_row * 3] = source;
+                state.unique_source_meta[out_row * 3 + 1] = token;
+                state.unique_source_meta[out_row * 3 + 2] = -1;
+            }
+        }
+        ++reads;
+        __threadfence();
+        fence_workgroup();
+        if (lane == 0) lds_store(q.rx_done + worker, ticket_index / state.rx_waves + 1);
+    }
+    if (lane == 0)
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatHostReads),
+                  static_cast<unsigned long long>(reads));
+}
+
+template <bool kFp8, bool kVector>
+__global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
+    __shared__ Queues q;
+    int entry_failed = 0;
+    if (threadIdx.x == 0) {
+        entry_failed = load_error_code(state) != 0;
+        q.abort = 0;
+        q.tx_finished = 0;
+        q.rx_finished = 0;
+        q.tx_head = 0;
+        q.rx_head = 0;
+        q.tx_total = -1;
+        q.rx_total = -1;
+        for (int i = 0; i < kMaxTxWaves; ++i) q.tx_done[i] = 0;
+        for (int i = 0; i < kMaxRxWaves; ++i) q.rx_done[i] = 0;
+    }
+    // One immutable entry verdict for the whole workgroup: branching on the
+    // mutable abort flag here could strand a wavefront at the final barrier
+    // (advanced_dispatch.cuh:935-938).
+    if (__syncthreads_or(entry_failed)) return;
+    const int channel = blockIdx.x;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (wave == 0) tx_control(state, q, channel, lane);
+    else if (wave == 1) rx_control(state, q, channel, lane);
+    else if (wave < 2 + state.tx_waves) tx_worker<kFp8, kVector>(state, q, channel, wave - 2, lane);
+    else rx_worker<kFp8, kVector>(state, q, channel, wave - 2 - state.tx_waves, lane);
+    // Every role loop has an explicit completion or abort exit; no workgroup
+    // barrier appears inside a role.
+    __syncthreads();
+    if (threadIdx.x == 0) state.channel_timestamps_ns[channel * 2 + 1] = ticks_to_ns(now_ticks());
+}
+
+}  // namespace
+
+int transport_threads(int tx_waves, int rx_waves) { return (2 + tx_waves + rx_waves) * kWave; }
+
+hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
+    const dim3 grid(state.z.dims.channels), block(transport_threads(state.tx_waves, state.rx_waves));
+    const bool fp8 = state.z.dims.wire_fp8 != 0;
+    // BF16 rows need 16-byte granularity on both sides; FP8 additionally needs
+    // whole 16-code vectors on the wire.
+    const bool vector = fp8 ? state.z.dims.hidden % 16 == 0 : state.z.dims.hidden % 8 == 0;
+    if (fp8 && vector) hipLaunchKernelGGL((transport_kernel<true, true>), grid, block, 0, stream, state);
+    else if (fp8) hipLaunchKernelGGL((transport_kernel<true, false>), grid, block, 0, stream, state);
+    else if (vector) hipLaunchKernelGGL((transport_kernel<false, true>), grid, block, 0, stream, state);
+    else hipLaunchKernelGGL((transport_kernel<false, false>), grid, block, 0, stream, state);
+    return hipGetLastError();
+}
+
+}  // namespace pcie_ep

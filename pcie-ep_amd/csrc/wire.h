@@ -1,0 +1,195 @@
+// Host-ring wire format shared by the gfx950 kernels and the host-side peer
+// emulator.  Plain C++ (no HIP types) so both sides compile it unchanged.
+//
+// One *segment* of pinned, fine-grained host memory exists per source rank.
+// Only the source writes payload slots, slot metadata, descriptor bodies,
+// READY words, the count mailbox, counts_ready, abort and channel_abort; a
+// receiver d writes only ack[..][d], the consumed word of its own (s -> d)
+// descriptor queue and counts_consumed[d].  Every 64-bit signal therefore has
+// exactly one writer and nothing ever performs a read-modify-write on host
+// memory (the discipline of the reference: csrc/kernels/host_staged/common.cuh:59-64).
+//
+// The byte layout is private to this build; it keeps the reference's protocol
+// objects (Signal / Descriptor / per-slot token metadata / count mailbox:
+// common.cuh:61-88, advanced_common.cuh:42-84) but
+//  * sizes the per-slot metadata by the runtime top-k instead of 32 branches,
+//  * stores it in the tail of the payload slot so one contiguous region is read,
+//  * groups the count mailbox by destination so a receiver reads one block.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define PCIE_EP_HD __host__ __device__ inline
+#else
+#define PCIE_EP_HD inline
+#endif
+
+namespace pcie_ep {
+
+constexpr int kMaxRanks = 16;      // common.cuh:12
+constexpr int kMaxTopk = 32;       // common.cuh:13
+constexpr int kMaxExperts = 4096;  // common.cuh:14
+constexpr int kMaxChannels = 32;   // pcie_ep/config.py:71
+constexpr int kErrorFields = 8;
+constexpr int kStatFields = 8;
+constexpr size_t kSignalBytes = 128;  // one writer per 128-byte line
+constexpr size_t kPageBytes = 4096;
+
+// Device error codes: values are part of the Python result contract
+// (csrc/kernels/host_staged/common.cuh:26-38).
+enum ErrorCode : int {
+    kOk = 0,
+    kErrInvalidRouting = 2,
+    kErrCountsMailboxWait = 11,
+    kErrCountsReadyWait = 12,
+    kErrBatchReadyWait = 13,
+    kErrBatchAckWait = 14,
+    kErrRingProgressWait = 15,
+    kErrExpandedCapacity = 16,
+    kErrPayloadSequence = 18,
+    kErrAlreadyAborted = 19,
+    kErrEpochExhausted = 20,
+};
+
+// stats[] fields (API.md:148 of the reference).
+enum StatField : int {
+    kStatHostWrites = 0,     // own tokens published to the host ring
+    kStatHostReads = 1,      // remote unique rows read from host rings
+    kStatDeliveries = 2,     // sum over published tokens of remote destination ranks
+    kStatMetaOverlap = 3,    // event counters, implementation specific
+    kStatRxNotReady = 4,
+    kStatTxCreditMiss = 5,
+    kStatTxStageBusy = 6,
+    kStatDescriptors = 7,    // endpoint descriptors published
+};
+
+struct alignas(128) Signal {
+    uint64_t value;
+    char pad[120];
+};
+
+// One entry of a (source -> destination, channel) notification queue.
+// Source writes everything except `consumed`; the destination writes `consumed`.
+struct alignas(128) Descriptor {
+    uint64_t ready;             // seq(epoch, ordinal) once the entry is complete
+    uint64_t payload_sequence;  // seq(epoch, token_index)
+    int32_t payload_slot;
+    int32_t token_index;
+    int32_t rank_ordinal;       // unique-row ordinal at this destination
+    int32_t reserved;
+    uint64_t consumed;          // seq(epoch, ordinal): credit returned by the destination
+    char pad[88];
+};
+static_assert(sizeof(Signal) == 128 && sizeof(Descriptor) == 128, "wire ABI");
+
+// Per-slot token metadata, stored after the payload bytes of the slot.
+//   header (32 B) | rank_ordinals[kMaxRanks] (64 B) | expert_indices[K] |
+//   expert_ordinals[K] | weights[K]
+struct SlotMetaHeader {
+    int32_t token_index;
+    uint32_t destination_mask;
+    float scale;  // FP8 per-token scale, 1.0 on a BF16 wire
+    int32_t reserved[5];
+};
+static_assert(sizeof(SlotMetaHeader) == 32, "wire ABI");
+constexpr int kMetaRankOrdinalsOffset = 32;
+constexpr int kMetaBranchOffset = 32 + 4 * kMaxRanks;  // 96
+
+PCIE_EP_HD size_t align_up(size_t value, size_t alignment) { return (value + alignment - 1) / alignment * alignment; }
+
+// `(epoch << 32) | (index + 1)`; zero means never written
+// (csrc/kernels/host_staged/advanced_common.cuh:203-205).
+PCIE_EP_HD uint64_t sequence(uint64_t epoch, int index) { return (epoch << 32) | uint64_t(uint32_t(index + 1)); }
+
+struct Dimensions {
+    int num_ranks;
+    int max_tokens;
+    int hidden;
+    int topk;
+    int num_experts;
+    int channels;
+    int payload_slots;     // Q, per channel
+    int descriptor_slots;  // L, per (channel, destination)
+    int wire_fp8;          // 0: BF16 payload, 1: E4M3FN payload + FP32 scale
+};
+
+struct SegmentLayout {
+    Dimensions dims;
+    int local_experts;
+    int payload_bytes;   // bytes of one row on the wire
+    int meta_offset;     // offset of the metadata inside a slot
+    int meta_bytes;      // 96 + 12*K rounded to 16
+    int mailbox_dwords;  // dwords of one per-destination mailbox block
+    size_t slot_stride;
+    size_t mailbox_stride;
+    size_t counts_ready_offset;
+    size_t counts_consumed_offset;  // [P] signals
+    size_t abort_offset;
+    size_t channel_abort_offset;    // [C] signals
+    size_t mailbox_offset;          // [P] blocks
+    size_t slots_offset;            // [C*Q] slots, page aligned
+    size_t ack_offset;              // [C*Q][P] signals
+    size_t descriptors_offset;      // [C][P][L] descriptors
+    size_t size_bytes;
+};
+
+// Mailbox block written by source s for destination d:
+//   dword 0: unique tokens s -> d;  dwords 1..EL: branches per local expert of d;
+//   dwords 1+EL .. 1+EL+C-1: unique tokens of each channel destined to d.
+PCIE_EP_HD SegmentLayout make_segment_layout(const Dimensions& dims) {
+    SegmentLayout z{};
+    z.dims = dims;
+    z.local_experts = dims.num_experts / dims.num_ranks;
+    z.payload_bytes = dims.hidden * (dims.wire_fp8 ? 1 : 2);
+    z.meta_offset = int(align_up(size_t(z.payload_bytes), 16));
+    z.meta_bytes = int(align_up(size_t(kMetaBranchOffset + 12 * dims.topk), 16));
+    z.slot_stride = align_up(size_t(z.meta_offset + z.meta_bytes), kPageBytes);
+    z.mailbox_dwords = 1 + z.local_experts + dims.channels;
+    z.mailbox_stride = align_up(size_t(z.mailbox_dwords) * 4, kSignalBytes);
+    size_t cursor = 0;
+    auto reserve = [&](size_t bytes) {
+        const size_t offset = cursor;
+        cursor += align_up(bytes, kSignalBytes);
+        return offset;
+    };
+    z.counts_ready_offset = reserve(sizeof(Signal));
+    z.counts_consumed_offset = reserve(size_t(dims.num_ranks) * sizeof(Signal));
+    z.abort_offset = reserve(sizeof(Signal));
+    z.channel_abort_offset = reserve(size_t(dims.channels) * sizeof(Signal));
+    z.mailbox_offset = reserve(size_t(dims.num_ranks) * z.mailbox_stride);
+    cursor = align_up(cursor, kPageBytes);
+    const size_t slots = size_t(dims.channels) * dims.payload_slots;
+    z.slots_offset = reserve(slots * z.slot_stride);
+    z.ack_offset = reserve(slots * dims.num_ranks * sizeof(Signal));
+    z.descriptors_offset = reserve(size_t(dims.channels) * dims.num_ranks * dims.descriptor_slots * sizeof(Descriptor));
+    z.size_bytes = align_up(cursor, kPageBytes);
+    return z;
+}
+
+PCIE_EP_HD uint64_t* signal_at(char* segment, size_t offset, size_t index = 0) {
+    return &reinterpret_cast<Signal*>(segment + offset)[index].value;
+}
+PCIE_EP_HD char* slot_at(const SegmentLayout& z, char* segment, int channel, int slot) {
+    return segment + z.slots_offset + (size_t(channel) * z.dims.payload_slots + slot) * z.slot_stride;
+}
+PCIE_EP_HD uint64_t* ack_at(const SegmentLayout& z, char* segment, int channel, int slot, int destination) {
+    return signal_at(segment, z.ack_offset, (size_t(channel) * z.dims.payload_slots + slot) * z.dims.num_ranks + destination);
+}
+PCIE_EP_HD Descriptor* descriptor_at(const SegmentLayout& z, char* segment, int channel, int destination, int ordinal) {
+    return reinterpret_cast<Descriptor*>(segment + z.descriptors_offset) +
+        (size_t(channel) * z.dims.num_ranks + destination) * z.dims.descriptor_slots + ordinal % z.dims.descriptor_slots;
+}
+PCIE_EP_HD int32_t* mailbox_at(const SegmentLayout& z, char* segment, int destination) {
+    return reinterpret_cast<int32_t*>(segment + z.mailbox_offset + size_t(destination) * z.mailbox_stride);
+}
+
+// Preallocated output capacities (csrc/buffers/advanced.hpp:296-298).
+PCIE_EP_HD int64_t unique_capacity(const Dimensions& d) { return int64_t(d.num_ranks) * d.max_tokens; }
+PCIE_EP_HD int64_t expanded_capacity(const Dimensions& d) {
+    const int local = d.num_experts / d.num_ranks;
+    return unique_capacity(d) * (d.topk < local ? d.topk : local) + int64_t(local) * 255;
+}
+
+}  // namespace pcie_ep

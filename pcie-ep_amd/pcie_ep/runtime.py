@@ -1,0 +1,241 @@
+"""Python half of the native runtime: result pools, route-plan pool and the call
+into ``pcie_ep_dispatch``.
+
+The C ABI takes raw device pointers, so tensor allocation and the ownership
+rules the reference implements inside its extension live here instead:
+
+* ``output_pool_size`` eager result pools plus one graph pool, all allocated at
+  construction (csrc/buffers/advanced.hpp:284-337); a pool is busy while any of
+  its tensors is referenced outside this module and an exhausted pool raises
+  instead of waiting or growing (advanced.hpp:402-418).
+* an equal number of route plans; a ``CachedLayout`` pins a plan, never a pool
+  (advanced.hpp:21-41, :131-147).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import itertools
+import sys
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from . import _native
+from .config import HostStagedConfig
+
+# Name, dtype and shape (in terms of the sizes below) of every pool tensor.
+_I32, _I64, _F32, _BF16 = torch.int32, torch.int64, torch.float32, torch.bfloat16
+
+_owner_ids = itertools.count(1)
+
+
+def _storage_uses(tensor: torch.Tensor) -> int:
+    return torch._C._storage_Use_Count(tensor.untyped_storage()._cdata)
+
+
+def _references(tensor: torch.Tensor) -> tuple:
+    return sys.getrefcount(tensor), _storage_uses(tensor)
+
+
+class RoutePlan:
+    """Opaque immutable routing state (the reference's ``_AdvancedLayout``)."""
+
+    def __init__(self, owner: int, nbytes: int, device: torch.device) -> None:
+        self.owner = owner
+        self.tokens = -1
+        self.storage = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+class _Pool:
+    def __init__(self, shapes: Dict[str, tuple], device: torch.device) -> None:
+        self.tensors: Dict[str, torch.Tensor] = {
+            name: torch.empty(shape, dtype=dtype, device=device) for name, (dtype, shape) in shapes.items()
+        }
+        self._idle = self._snapshot()
+
+    def _snapshot(self) -> list:
+        return [_references(self.tensors[name]) for name in self.tensors]
+
+    def idle(self) -> bool:
+        """True while nothing outside this pool references any of its tensors
+        (Python objects or views of their storage)."""
+        return self._snapshot() == self._idle
+
+
+class NativeRuntime:
+    """Owns one ``pcie_ep_runtime`` plus its preallocated pools."""
+
+    def __init__(self, rank: int, world: int, max_tokens: int, hidden: int, topk: int, experts: int, config: HostStagedConfig,
+                 device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0) -> None:
+        self._lib = _native.library()
+        self.config = config
+        self.device = torch.device("cuda", device)
+        self.owner_id = next(_owner_ids)
+        native = _native.Config(
+            num_ranks=world, local_rank=rank, max_tokens=max_tokens, hidden=hidden, topk=topk, num_experts=experts,
+            channels=config.channels, payload_slots=config.payload_slots, descriptor_slots=config.descriptor_slots,
+            wire_fp8=int(config.wire_dtype == "fp8_e4m3"), timeout_ms=config.timeout_ms,
+            fuse_receive_expand=int(config.fuse_receive_expand), tx_waves=tx_waves, rx_waves=rx_waves,
+            peer_threads=peer_threads, staging_numa_node=staging_numa_node, device=device,
+        )
+        self.native_config = native
+        self.sizes = _native.Sizes()
+        _native.check(self._lib.pcie_ep_query_sizes(C.byref(native), C.byref(self.sizes)), invalid=RuntimeError)
+        handle = C.c_void_p()
+        _native.check(self._lib.pcie_ep_runtime_create(C.byref(native), C.byref(handle)), invalid=RuntimeError)
+        self._handle: Optional[C.c_void_p] = handle
+        self.world, self.rank, self.hidden, self.topk = world, rank, hidden, topk
+        self.max_tokens, self.experts = max_tokens, experts
+        self.channels = config.channels
+        try:
+            self._allocate()
+            self._lib.pcie_ep_set_test_delays(handle, config.metadata_delay_ns, config.tx_delay_ns, config.rx_delay_ns,
+                                              config.scatter_delay_ns)
+        except Exception:
+            self.close()
+            raise
+
+    # ---- allocation -----------------------------------------------------------------
+    def _allocate(self) -> None:
+        n, capacity = int(self.sizes.unique_rows), int(self.sizes.expanded_rows)
+        h, k, p, local, c = self.hidden, self.topk, self.world, int(self.sizes.local_experts), self.channels
+        shapes = {
+            "unique_payload": (_BF16, (n, h)), "unique_topk_idx": (_I64, (n, k)), "unique_topk_weights": (_F32, (n, k)),
+            "unique_source_meta": (_I64, (n, 3)), "unique_expert_ordinals": (_I32, (n, k)),
+            "expanded_payload": (_BF16, (capacity, h)), "expanded_expert_idx": (_I64, (capacity,)),
+            "expanded_weights": (_F32, (capacity,)), "expanded_source_meta": (_I64, (capacity, 3)),
+            "unique_count": (_I64, (1,)), "expanded_count": (_I64, (1,)), "expert_prefix": (_I32, (local,)),
+            "expert_counts": (_I32, (local,)), "expert_offsets": (_I32, (local + 1,)), "source_offsets": (_I32, (p + 1,)),
+            "source_expert_prefix": (_I32, (p, local)), "errors": (_I64, (8,)), "stats": (_I64, (8,)),
+            "transport_timestamps_ns": (_I64, (2,)), "expected_receive_counts": (_I32, (c, p)),
+            "channel_stats": (_I64, (c, 8)), "channel_timestamps_ns": (_I64, (c, 2)),
+            "receive_expand_overlap": (_I64, (c, 2)), "receive_prefix_state": (_I64, (2,)),
+            "prefix_tx_timestamps_ns": (_I64, (c + 1, 2)),
+        }
+        assert tuple(shapes) == _native.OUTPUT_POINTERS
+        eager = self.config.output_pool_size
+        self._pools: List[_Pool] = [_Pool(shapes, self.device) for _ in range(eager + int(self.config.enable_graph))]
+        self._plans: List[RoutePlan] = [RoutePlan(self.owner_id, int(self.sizes.plan_bytes), self.device) for _ in range(eager)]
+        self._graph_plan = RoutePlan(self.owner_id, int(self.sizes.plan_bytes), self.device) if self.config.enable_graph else None
+        self._plan_idle = self._plan_references(0)
+
+    def _plan_references(self, index: int) -> int:
+        return sys.getrefcount(self._plans[index])
+
+    # ---- dispatch ---------------------------------------------------------------------
+    def _select_pool(self, graph_pool: bool) -> _Pool:
+        if graph_pool:
+            if not self.config.enable_graph:
+                raise RuntimeError("Graph output pool was not prepared")
+            return self._pools[self.config.output_pool_size]
+        for pool in self._pools[: self.config.output_pool_size]:
+            if pool.idle():
+                return pool
+        raise RuntimeError("preallocated output pool exhausted; release prior results or use a separate buffer")
+
+    def _select_plan(self, tokens: int, cached_layout: Optional[RoutePlan], graph_pool: bool) -> RoutePlan:
+        if cached_layout is not None:
+            if not isinstance(cached_layout, RoutePlan) or cached_layout.owner != self.owner_id or cached_layout.tokens != tokens:
+                raise RuntimeError("cached route layout belongs to another buffer or input shape")
+            return cached_layout
+        if graph_pool:
+            assert self._graph_plan is not None
+            self._graph_plan.tokens = tokens
+            return self._graph_plan
+        for index in range(len(self._plans)):
+            if self._plan_references(index) == self._plan_idle:
+                self._plans[index].tokens = tokens
+                return self._plans[index]
+        raise RuntimeError("preallocated route plan pool exhausted; release old handles/cache plans")
+
+    def dispatch(self, x: torch.Tensor, idx: torch.Tensor, weights: Optional[torch.Tensor], stage: int, alignment: int,
+                 expand: bool, zero_padding: bool, cached_layout: Any = None, graph_pool: bool = False) -> Dict[str, Any]:
+        """Enqueue one dispatch on the current stream and return the result dict
+        (counterpart of ``AdvancedRuntime.dispatch``: advanced.hpp:126-156)."""
+        if self._handle is None:
+            raise RuntimeError("advanced runtime is closed or closing")
+        if stage != self.config.stage:
+            raise RuntimeError("advanced stage differs from prepared configuration")
+        if not 1 <= alignment <= 256:
+            raise RuntimeError("alignment must be in [1,256]")
+        pool = self._select_pool(graph_pool)
+        plan = self._select_plan(int(x.shape[0]), cached_layout, graph_pool)
+        arguments = _native.DispatchArgs(
+            x=x.data_ptr(), topk_idx=idx.data_ptr(), topk_weights=weights.data_ptr() if weights is not None else None,
+            num_tokens=int(x.shape[0]), alignment=alignment, expand=int(expand), zero_padding=int(zero_padding),
+            reuse_plan=int(cached_layout is not None), plan=plan.storage.data_ptr(),
+            expanded_capacity_rows=int(self.sizes.expanded_rows),
+            **{name: pool.tensors[name].data_ptr() for name in _native.OUTPUT_POINTERS},
+        )
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _native.check(self._lib.pcie_ep_dispatch(self._handle, C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
+        t = pool.tensors
+        fused = bool(expand and self.config.fuse_receive_expand)
+        result: Dict[str, Any] = {
+            "recv_x": t["expanded_payload"] if expand else t["unique_payload"],
+            "recv_topk_idx": t["expanded_expert_idx"] if expand else t["unique_topk_idx"],
+            "recv_topk_weights": t["expanded_weights"] if expand else t["unique_topk_weights"],
+            "source_meta": t["expanded_source_meta"] if expand else t["unique_source_meta"],
+            "receive_expand_overlap": t["receive_expand_overlap"] if fused and self.config.receive_expand_mode != "scalar" else None,
+            "unique_count": t["unique_count"], "expanded_count": t["expanded_count"], "expert_prefix": t["expert_prefix"],
+            "expert_counts": t["expert_counts"], "expert_offsets": t["expert_offsets"], "source_offsets": t["source_offsets"],
+            "error": t["errors"], "stats": t["stats"], "transport_timestamps_ns": t["transport_timestamps_ns"],
+            "channel_stats": t["channel_stats"], "channel_timestamps_ns": t["channel_timestamps_ns"],
+            "prefix_tx_timestamps_ns": t["prefix_tx_timestamps_ns"],
+            "_layout": None if (graph_pool and cached_layout is None) else plan,
+        }
+        return result
+
+    # ---- diagnostics and hooks ----------------------------------------------------------
+    def pool_debug(self) -> list:
+        return [[_references(tensor) for tensor in pool.tensors.values()] for pool in self._pools]
+
+    def _require(self) -> C.c_void_p:
+        if self._handle is None:
+            raise RuntimeError("advanced runtime is closed or closing")
+        return self._handle
+
+    def set_test_delays(self, metadata_ns: int, tx_ns: int, rx_ns: int, scatter_ns: int) -> None:
+        _native.check(self._lib.pcie_ep_set_test_delays(self._require(), metadata_ns, tx_ns, rx_ns, scatter_ns))
+
+    def set_test_prefix_delay_ns(self, delay_ns: int) -> None:
+        _native.check(self._lib.pcie_ep_set_test_prefix_delay_ns(self._require(), delay_ns))
+
+    def set_test_control_abort_after_ns(self, delay_ns: int) -> None:
+        _native.check(self._lib.pcie_ep_set_test_control_abort_after_ns(self._require(), delay_ns))
+
+    def set_test_skip_counts_ack_source(self, source: int) -> None:
+        _native.check(self._lib.pcie_ep_set_test_skip_counts_ack_source(self._require(), source), invalid=RuntimeError)
+
+    def host_signal_store(self, segment_rank: int, which: int, index: int, value: int) -> None:
+        _native.check(self._lib.pcie_ep_host_signal_store(self._require(), segment_rank, which, index, value))
+
+    def host_signal_load(self, segment_rank: int, which: int, index: int) -> int:
+        value = C.c_uint64()
+        _native.check(self._lib.pcie_ep_host_signal_load(self._require(), segment_rank, which, index, C.byref(value)))
+        return int(value.value)
+
+    def expand_unique(self, pool_tensors: Dict[str, torch.Tensor], plan: RoutePlan, alignment: int, zero_padding: bool) -> None:
+        """Run only the stand-alone expand kernel on an existing result (benchmarks)."""
+        arguments = _native.DispatchArgs(
+            x=None, topk_idx=None, topk_weights=None, num_tokens=0, alignment=alignment, expand=1,
+            zero_padding=int(zero_padding), reuse_plan=1, plan=plan.storage.data_ptr(),
+            expanded_capacity_rows=int(self.sizes.expanded_rows),
+            **{name: pool_tensors[name].data_ptr() for name in _native.OUTPUT_POINTERS},
+        )
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _native.check(self._lib.pcie_ep_expand_unique(self._require(), C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
+
+    def pool_tensors(self, index: int) -> Dict[str, torch.Tensor]:
+        return self._pools[index].tensors
+
+    @property
+    def handle(self) -> C.c_void_p:
+        return self._require()
+
+    def close(self) -> None:
+        if self._handle is None:
+            return
+        handle, self._handle = self._handle, None
+        _native.check(self._lib.pcie_ep_runtime_destroy(handle), invalid=RuntimeError)

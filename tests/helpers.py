@@ -1,0 +1,215 @@
+"""Workload generators and the result checker shared by the GPU parity tests.
+
+The checker compares every output of ``HostStagedEPBuffer.dispatch`` with the
+CPU oracle (``oracle/``), bit for bit: counts, offsets, prefixes, row payloads,
+expert ids, weights, source metadata, padding and the deterministic statistics.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from oracle import dispatch_oracle as oracle
+from oracle import fp8_oracle
+
+Inputs = Tuple[torch.Tensor, torch.Tensor, torch.Tensor]  # x bf16 [T,H], idx int64 [T,K], weights f32 [T,K]
+
+
+def payload_pattern(source: int, tokens: int, hidden: int) -> torch.Tensor:
+    """Finite BF16 rows whose raw bits are a hash of (source, token, column), so a
+    misrouted or torn row identifies itself (idea of tests/test_large.py:34-43 of
+    the reference; a different mixer).  Exponent field 16..235, both signs."""
+    token = np.arange(tokens, dtype=np.uint64)[:, None]
+    column = np.arange(hidden, dtype=np.uint64)[None, :]
+    key = np.uint64(source + 1) * np.uint64(0x9E3779B97F4A7C15) + token * np.uint64(0xC2B2AE3D27D4EB4F) + column * np.uint64(0x165667B19E3779F9)
+    key ^= key >> np.uint64(29)
+    key *= np.uint64(0xBF58476D1CE4E5B9)
+    key ^= key >> np.uint64(32)
+    mantissa = key & np.uint64(0x7F)
+    exponent = (key >> np.uint64(7)) % np.uint64(220) + np.uint64(16)
+    sign = (key >> np.uint64(40)) & np.uint64(1)
+    bits = (mantissa | (exponent << np.uint64(7)) | (sign << np.uint64(15))).astype(np.uint16)
+    return torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+
+
+def make_routes(generator: torch.Generator, tokens: int, experts: int, topk: int, pattern: str, rank: int, world: int) -> torch.Tensor:
+    """Route patterns of the reference's correctness matrix (tests/test_correctness.py:31-57)."""
+    local = experts // world
+    if pattern == "local":
+        idx = (torch.arange(topk) + rank * local).repeat(tokens, 1)
+    elif pattern == "multicast":
+        ids = [dest * local + e for e in range(local) for dest in range(world)]
+        idx = torch.tensor(ids[:topk], dtype=torch.int64).repeat(tokens, 1)
+    elif pattern == "hotspot":
+        idx = torch.arange(topk).repeat(tokens, 1)
+    else:
+        idx = torch.rand(tokens, experts, generator=generator).topk(topk, dim=1).indices
+    idx = idx.to(torch.int64).clone()
+    if pattern == "none":
+        idx.fill_(-1)
+    elif pattern == "partial" and tokens:
+        idx[:, ::3] = -1
+    return idx.reshape(tokens, topk).contiguous()
+
+
+def make_inputs(world: int, tokens: Sequence[int], hidden: int, experts: int, topk: int, pattern: str = "random", seed: int = 7,
+                gaussian: bool = False, heavy_tail: bool = False) -> List[Inputs]:
+    inputs = []
+    for rank in range(world):
+        generator = torch.Generator().manual_seed(seed + rank * 7919)
+        count = tokens[rank]
+        idx = make_routes(generator, count, experts, topk, pattern, rank, world)
+        weights = torch.softmax(torch.randn(count, topk, generator=generator), dim=1).to(torch.float32).contiguous()
+        if gaussian:
+            x = torch.randn(count, hidden, generator=generator)
+            if heavy_tail:
+                channels = torch.randperm(hidden, generator=torch.Generator().manual_seed(seed))[: max(1, hidden // 100)]
+                x[:, channels] *= 50.0
+            x = x.to(torch.bfloat16)
+        else:
+            x = payload_pattern(rank, count, hidden)
+        inputs.append((x.contiguous(), idx, weights))
+    return inputs
+
+
+def _bits(tensor: torch.Tensor) -> np.ndarray:
+    return tensor.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def expected_rows(inputs: Sequence[Inputs], rank: int, fp8_wire: bool) -> List[np.ndarray]:
+    """BF16 bit rows each source delivers to ``rank``: the original for the
+    local source, the FP8 round trip for remote sources on an FP8 wire
+    (tests/test_s7.py:154-157 of the reference)."""
+    rows = []
+    for source, (x, _, _) in enumerate(inputs):
+        if fp8_wire and source != rank and x.shape[0]:
+            rows.append(_bits(fp8_oracle.roundtrip(x)))
+        else:
+            rows.append(_bits(x))
+    return rows
+
+
+def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, experts: int, topk: int, expand: bool, alignment: int,
+                    zero_padding: bool, with_weights: bool = True, fp8_wire: bool = False, check_stats: bool = True) -> dict:
+    recv_x, recv_idx, recv_weights, handle, event = result
+    event.current_stream_wait()
+    torch.cuda.synchronize()
+    error = handle.error.cpu().tolist()
+    assert not any(error), f"GPU error {error}"
+    all_idx = [idx.numpy() for _, idx, _ in inputs]
+    expectation = oracle.expected_dispatch(all_idx, rank, world, experts, alignment)
+    receiver = expectation.receiver
+    assert int(handle.unique_count.cpu()) == receiver.unique_count
+    assert int(handle.expanded_count.cpu()) == receiver.expanded_count
+    assert handle.expert_counts.cpu().numpy().tolist() == receiver.expert_counts.tolist()
+    assert handle.expert_offsets.cpu().numpy().tolist() == receiver.expert_offsets.tolist()
+    assert handle.psum_num_recv_tokens_per_expert.cpu().numpy().tolist() == receiver.expert_prefix.tolist()
+    assert handle.source_offsets.cpu().numpy().tolist() == receiver.source_offsets.tolist()
+    assert handle.psum_num_recv_tokens_per_scaleup_rank.cpu().numpy().tolist() == receiver.source_offsets[1:].tolist()
+    rows = expected_rows(inputs, rank, fp8_wire)
+    weights_in = [w.numpy() for _, _, w in inputs]
+    meta = handle.source_meta.cpu().numpy()
+    if with_weights:
+        assert recv_weights is not None
+    else:
+        assert recv_weights is None
+    if expand:
+        e = expectation.expanded
+        out_rows = torch.from_numpy(e.rows)
+        got = _bits(recv_x[out_rows.to(recv_x.device)]) if e.rows.size else np.zeros((0, recv_x.shape[1]), np.uint16)
+        want = np.zeros_like(got)
+        want_weights = np.zeros(e.rows.size, np.float32)
+        for source in range(world):
+            select = e.source == source
+            want[select] = rows[source][e.token[select]]
+            want_weights[select] = weights_in[source][e.token[select], e.branch[select]]
+        assert np.array_equal(got, want), "expanded payload rows differ"
+        idx_out = recv_idx.cpu().numpy()
+        assert np.array_equal(idx_out[e.rows], e.expert.astype(np.int64)), "expanded expert ids differ"
+        assert np.array_equal(meta[e.rows], np.stack([e.source, e.token, e.branch], axis=1).astype(np.int64)), "expanded source_meta differs"
+        if with_weights:
+            got_weights = recv_weights.cpu().numpy()[e.rows]
+            assert np.array_equal(got_weights.view(np.uint32), want_weights.view(np.uint32)), "expanded weights differ"
+        if zero_padding and e.padding_rows.size:
+            pad = torch.from_numpy(e.padding_rows).to(recv_x.device)
+            assert not torch.count_nonzero(recv_x[pad].view(torch.int16)), "payload padding is not zero"
+            assert (idx_out[e.padding_rows] == -1).all(), "index padding is not -1"
+            assert (meta[e.padding_rows] == -1).all(), "metadata padding is not -1"
+            if with_weights:
+                assert not np.count_nonzero(recv_weights.cpu().numpy()[e.padding_rows]), "weight padding is not zero"
+    else:
+        u = expectation.unique
+        assert sorted(u.rows.tolist()) == list(range(receiver.unique_count))
+        out_rows = torch.from_numpy(u.rows)
+        got = _bits(recv_x[out_rows.to(recv_x.device)]) if u.rows.size else np.zeros((0, recv_x.shape[1]), np.uint16)
+        want = np.zeros_like(got)
+        want_weights = np.zeros((u.rows.size, topk), np.float32)
+        for source in range(world):
+            select = u.source == source
+            want[select] = rows[source][u.token[select]]
+            want_weights[select] = np.where(u.topk_mask[select], weights_in[source][u.token[select]], 0.0)
+        assert np.array_equal(got, want), "unique payload rows differ"
+        assert np.array_equal(recv_idx.cpu().numpy()[u.rows], u.topk_idx), "unique routes differ"
+        assert np.array_equal(meta[u.rows][:, :2], np.stack([u.source, u.token], axis=1).astype(np.int64)), "unique identity differs"
+        assert (meta[u.rows][:, 2] == -1).all()
+        if with_weights:
+            got_weights = recv_weights.cpu().numpy()[u.rows]
+            assert np.array_equal(got_weights.view(np.uint32), want_weights.view(np.uint32)), "unique weights differ"
+    stats = handle.stats.cpu().numpy()
+    if check_stats:
+        for field in (0, 1, 2, 7):
+            assert int(stats[field]) == int(expectation.stats[field]), f"stats[{field}] = {int(stats[field])}, expected {int(expectation.stats[field])}"
+    return {"unique": receiver.unique_count, "expanded": receiver.expanded_count, "stats": stats.tolist()}
+
+
+def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, experts: int, topk: int, fp8_wire: bool = False) -> int:
+    """TX parity: what every emulated receiver got from the GPU must be exactly
+    the GPU source's unique rows for that receiver (payload bytes, ordinals,
+    global expert ids, live weights), each row once."""
+    x, idx, weights = inputs[gpu_rank]
+    layout = oracle.source_layout(idx.numpy(), world, experts)
+    total = 0
+    if fp8_wire and x.shape[0]:
+        codes, scales = fp8_oracle.quantize(x)
+        wire, wire_scales = codes.numpy(), scales.numpy()
+    else:
+        wire, wire_scales = _bits(x).view(np.uint8).reshape(x.shape[0], -1), np.ones(x.shape[0], np.float32)
+    for rank in range(world):
+        if rank == gpu_rank:
+            continue
+        got = peers.captured(rank)
+        want_tokens = np.nonzero((layout.destination_mask >> np.uint64(rank)) & np.uint64(1))[0]
+        order = np.argsort(got["tokens"], kind="stable")
+        assert np.array_equal(got["tokens"][order], want_tokens), f"rank {rank} received the wrong token set"
+        tokens = got["tokens"][order]
+        assert np.array_equal(got["rank_ordinals"][order], layout.rank_ordinals[tokens, rank])
+        assert np.array_equal(got["masks"][order].astype(np.uint64), layout.destination_mask[tokens])
+        assert np.array_equal(got["expert_idx"][order], layout.expert_indices[tokens])
+        assert np.array_equal(got["expert_ordinals"][order], layout.expert_ordinals[tokens])
+        assert np.array_equal(got["weights"][order].view(np.uint32), weights.numpy()[tokens].view(np.uint32))
+        assert np.array_equal(got["payload"][order], wire[tokens]), f"rank {rank} received different payload bytes"
+        assert np.array_equal(got["scales"][order].view(np.uint32), wire_scales[tokens].view(np.uint32))
+        total += tokens.size
+    return total
+
+
+def run_dispatch(buffer, inputs: Sequence[Inputs], expand: bool = True, alignment: int = 1, zero_padding: bool = False,
+                 with_weights: bool = True, capture: bool = False, handle=None, peers_already_set: bool = False, **kwargs):
+    """Arm the peers for one epoch, dispatch the GPU rank's inputs, wait for the peers."""
+    rank = buffer.rank_idx
+    if buffer.peers is not None:
+        if not peers_already_set:
+            for source, (x, idx, weights) in enumerate(inputs):
+                if source != rank:
+                    buffer.peers.set_source(source, x, idx, weights if with_weights else None)
+        buffer.peers.start(1, capture=capture)
+    x, idx, weights = (item.cuda() for item in inputs[rank])
+    result = buffer.dispatch(x, topk_idx=None if handle is not None else idx, topk_weights=weights if with_weights else None,
+                             do_expand=expand, expert_alignment=alignment, do_zero_padding=zero_padding, handle=handle, **kwargs)
+    torch.cuda.synchronize()
+    if buffer.peers is not None:
+        buffer.peers.wait(30_000)
+    return result, (x, idx, weights)
