@@ -371,13 +371,14 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
                 const int token = list[cursor];
                 if ((state.mask[token] >> me_) & 1u) {
                     const int slot = cursor % slots;
-                    if (cursor >= slots) {
-                        const int previous = list[cursor - slots];
-                        if (((state.mask[previous] >> me_) & 1u) &&
-                            acquire(ack_at(z_, own, channel, slot, me_)) != sequence(epoch, previous))
-                            break;
-                        // The previous occupant is retired; the slot is re-listed when it is published again.
-                        state.pending_sequence[size_t(channel) * slots + slot] = 0;
+                    // The slot may be rewritten only after the GPU ACKed the last row
+                    // that was published to it here.  Occupants bound for other
+                    // emulated ranks are never written, so the previous ring
+                    // occupant is not necessarily the one whose ACK matters.
+                    const size_t slot_index = size_t(channel) * slots + slot;
+                    if (state.pending_sequence[slot_index]) {
+                        if (acquire(ack_at(z_, own, channel, slot, me_)) != state.pending_sequence[slot_index]) break;
+                        state.pending_sequence[slot_index] = 0;
                     }
                     const int ordinal = state.sent[channel];
                     if (ordinal >= descriptors &&

@@ -18,21 +18,21 @@ from oracle import fp8_oracle
 Inputs = Tuple[torch.Tensor, torch.Tensor, torch.Tensor]  # x bf16 [T,H], idx int64 [T,K], weights f32 [T,K]
 
 
-def payload_pattern(source: int, tokens: int, hidden: int) -> torch.Tensor:
+def payload_pattern(source: int, tokens: int, hidden: int, device: str = "cpu") -> torch.Tensor:
     """Finite BF16 rows whose raw bits are a hash of (source, token, column), so a
     misrouted or torn row identifies itself (idea of tests/test_large.py:34-43 of
     the reference; a different mixer).  Exponent field 16..235, both signs."""
-    token = np.arange(tokens, dtype=np.uint64)[:, None]
-    column = np.arange(hidden, dtype=np.uint64)[None, :]
-    key = np.uint64(source + 1) * np.uint64(0x9E3779B97F4A7C15) + token * np.uint64(0xC2B2AE3D27D4EB4F) + column * np.uint64(0x165667B19E3779F9)
-    key ^= key >> np.uint64(29)
-    key *= np.uint64(0xBF58476D1CE4E5B9)
-    key ^= key >> np.uint64(32)
-    mantissa = key & np.uint64(0x7F)
-    exponent = (key >> np.uint64(7)) % np.uint64(220) + np.uint64(16)
-    sign = (key >> np.uint64(40)) & np.uint64(1)
-    bits = (mantissa | (exponent << np.uint64(7)) | (sign << np.uint64(15))).astype(np.uint16)
-    return torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    token = torch.arange(tokens, dtype=torch.int64, device=device).view(-1, 1)
+    column = torch.arange(hidden, dtype=torch.int64, device=device).view(1, -1)
+    key = (source + 1) * 0x3C6EF372 + token * 0x27D4EB2F + column * 0x165667B1
+    key = (key ^ (key >> 15)) * 0x2C1B3C6D
+    key = (key ^ (key >> 12)) * 0x297A2D39
+    key = (key ^ (key >> 15)) & 0xFFFFFFFF
+    mantissa = key & 0x7F
+    exponent = (((key >> 7) & 0xFFFF) * 220 >> 16) + 16
+    sign = (key >> 24) & 1
+    bits = mantissa | (exponent << 7) | (sign << 15)
+    return bits.to(torch.int16).view(torch.bfloat16).cpu().contiguous()
 
 
 def make_routes(generator: torch.Generator, tokens: int, experts: int, topk: int, pattern: str, rank: int, world: int) -> torch.Tensor:
@@ -70,7 +70,7 @@ def make_inputs(world: int, tokens: Sequence[int], hidden: int, experts: int, to
                 x[:, channels] *= 50.0
             x = x.to(torch.bfloat16)
         else:
-            x = payload_pattern(rank, count, hidden)
+            x = payload_pattern(rank, count, hidden, "cuda" if torch.cuda.is_available() else "cpu")
         inputs.append((x.contiguous(), idx, weights))
     return inputs
 
@@ -79,17 +79,28 @@ def _bits(tensor: torch.Tensor) -> np.ndarray:
     return tensor.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
-def expected_rows(inputs: Sequence[Inputs], rank: int, fp8_wire: bool) -> List[np.ndarray]:
-    """BF16 bit rows each source delivers to ``rank``: the original for the
-    local source, the FP8 round trip for remote sources on an FP8 wire
+def expected_bank(inputs: Sequence[Inputs], rank: int, fp8_wire: bool, device) -> Tuple[torch.Tensor, np.ndarray]:
+    """All rows every source can deliver to ``rank`` as one int16 [sum T, H]
+    tensor on ``device`` plus each source's first row: the original BF16 bits for
+    the local source, the FP8 round trip for remote sources on an FP8 wire
     (tests/test_s7.py:154-157 of the reference)."""
-    rows = []
+    parts, base, cursor = [], [], 0
     for source, (x, _, _) in enumerate(inputs):
-        if fp8_wire and source != rank and x.shape[0]:
-            rows.append(_bits(fp8_oracle.roundtrip(x)))
-        else:
-            rows.append(_bits(x))
-    return rows
+        rows = fp8_oracle.roundtrip(x) if (fp8_wire and source != rank and x.shape[0]) else x
+        parts.append(rows.contiguous().view(torch.int16).to(device))
+        base.append(cursor)
+        cursor += x.shape[0]
+    return torch.cat(parts), np.asarray(base, dtype=np.int64)
+
+
+def _rows_equal(recv_x: torch.Tensor, out_rows: np.ndarray, bank: torch.Tensor, bank_rows: np.ndarray, chunk: int = 16384) -> bool:
+    got_all = recv_x.view(torch.int16)
+    for begin in range(0, out_rows.size, chunk):
+        rows = torch.from_numpy(out_rows[begin : begin + chunk]).to(recv_x.device)
+        want = torch.from_numpy(bank_rows[begin : begin + chunk]).to(recv_x.device)
+        if not torch.equal(got_all[rows], bank[want]):
+            return False
+    return True
 
 
 def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, experts: int, topk: int, expand: bool, alignment: int,
@@ -109,7 +120,7 @@ def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, exp
     assert handle.psum_num_recv_tokens_per_expert.cpu().numpy().tolist() == receiver.expert_prefix.tolist()
     assert handle.source_offsets.cpu().numpy().tolist() == receiver.source_offsets.tolist()
     assert handle.psum_num_recv_tokens_per_scaleup_rank.cpu().numpy().tolist() == receiver.source_offsets[1:].tolist()
-    rows = expected_rows(inputs, rank, fp8_wire)
+    bank, base = expected_bank(inputs, rank, fp8_wire, recv_x.device)
     weights_in = [w.numpy() for _, _, w in inputs]
     meta = handle.source_meta.cpu().numpy()
     if with_weights:
@@ -118,15 +129,11 @@ def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, exp
         assert recv_weights is None
     if expand:
         e = expectation.expanded
-        out_rows = torch.from_numpy(e.rows)
-        got = _bits(recv_x[out_rows.to(recv_x.device)]) if e.rows.size else np.zeros((0, recv_x.shape[1]), np.uint16)
-        want = np.zeros_like(got)
+        assert _rows_equal(recv_x, e.rows, bank, base[e.source] + e.token), "expanded payload rows differ"
         want_weights = np.zeros(e.rows.size, np.float32)
         for source in range(world):
             select = e.source == source
-            want[select] = rows[source][e.token[select]]
             want_weights[select] = weights_in[source][e.token[select], e.branch[select]]
-        assert np.array_equal(got, want), "expanded payload rows differ"
         idx_out = recv_idx.cpu().numpy()
         assert np.array_equal(idx_out[e.rows], e.expert.astype(np.int64)), "expanded expert ids differ"
         assert np.array_equal(meta[e.rows], np.stack([e.source, e.token, e.branch], axis=1).astype(np.int64)), "expanded source_meta differs"
@@ -143,15 +150,11 @@ def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, exp
     else:
         u = expectation.unique
         assert sorted(u.rows.tolist()) == list(range(receiver.unique_count))
-        out_rows = torch.from_numpy(u.rows)
-        got = _bits(recv_x[out_rows.to(recv_x.device)]) if u.rows.size else np.zeros((0, recv_x.shape[1]), np.uint16)
-        want = np.zeros_like(got)
+        assert _rows_equal(recv_x, u.rows, bank, base[u.source] + u.token), "unique payload rows differ"
         want_weights = np.zeros((u.rows.size, topk), np.float32)
         for source in range(world):
             select = u.source == source
-            want[select] = rows[source][u.token[select]]
             want_weights[select] = np.where(u.topk_mask[select], weights_in[source][u.token[select]], 0.0)
-        assert np.array_equal(got, want), "unique payload rows differ"
         assert np.array_equal(recv_idx.cpu().numpy()[u.rows], u.topk_idx), "unique routes differ"
         assert np.array_equal(meta[u.rows][:, :2], np.stack([u.source, u.token], axis=1).astype(np.int64)), "unique identity differs"
         assert (meta[u.rows][:, 2] == -1).all()
@@ -165,7 +168,8 @@ def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, exp
     return {"unique": receiver.unique_count, "expanded": receiver.expanded_count, "stats": stats.tolist()}
 
 
-def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, experts: int, topk: int, fp8_wire: bool = False) -> int:
+def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, experts: int, topk: int, fp8_wire: bool = False,
+                    with_weights: bool = True) -> int:
     """TX parity: what every emulated receiver got from the GPU must be exactly
     the GPU source's unique rows for that receiver (payload bytes, ordinals,
     global expert ids, live weights), each row once."""
@@ -176,7 +180,7 @@ def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, 
         codes, scales = fp8_oracle.quantize(x)
         wire, wire_scales = codes.numpy(), scales.numpy()
     else:
-        wire, wire_scales = _bits(x).view(np.uint8).reshape(x.shape[0], -1), np.ones(x.shape[0], np.float32)
+        wire, wire_scales = _bits(x).view(np.uint8).reshape(x.shape[0], x.shape[1] * 2), np.ones(x.shape[0], np.float32)
     for rank in range(world):
         if rank == gpu_rank:
             continue
@@ -189,7 +193,8 @@ def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, 
         assert np.array_equal(got["masks"][order].astype(np.uint64), layout.destination_mask[tokens])
         assert np.array_equal(got["expert_idx"][order], layout.expert_indices[tokens])
         assert np.array_equal(got["expert_ordinals"][order], layout.expert_ordinals[tokens])
-        assert np.array_equal(got["weights"][order].view(np.uint32), weights.numpy()[tokens].view(np.uint32))
+        sent = weights.numpy()[tokens] if with_weights else np.ones((tokens.size, topk), np.float32)  # 1.0 without weights
+        assert np.array_equal(got["weights"][order].view(np.uint32), sent.view(np.uint32))
         assert np.array_equal(got["payload"][order], wire[tokens]), f"rank {rank} received different payload bytes"
         assert np.array_equal(got["scales"][order].view(np.uint32), wire_scales[tokens].view(np.uint32))
         total += tokens.size
@@ -211,5 +216,9 @@ def run_dispatch(buffer, inputs: Sequence[Inputs], expand: bool = True, alignmen
                              do_expand=expand, expert_alignment=alignment, do_zero_padding=zero_padding, handle=handle, **kwargs)
     torch.cuda.synchronize()
     if buffer.peers is not None:
-        buffer.peers.wait(30_000)
+        try:
+            buffer.peers.wait(30_000)
+        except Exception as exc:
+            raise AssertionError(f"peer emulator failed ({exc}); GPU error field {result[3].error.cpu().tolist()}, "
+                                 f"stats {result[3].stats.cpu().tolist()}") from exc
     return result, (x, idx, weights)

@@ -1,5 +1,14 @@
 """GPU parity of the full dispatch against the CPU oracle (bit-exact), through
-the drop-in Python surface and therefore through the C ABI."""
+the drop-in Python surface and therefore through the C ABI.
+
+The matrix follows the reference's distributed correctness test
+(tests/test_correctness.py:228-262): ring windows Q/L in {(1,1),(2,3),(3,2),
+(256,256)}, route patterns random / local / multicast / hotspot / partial /
+none, unique and expanded layouts, T in {0, 17, 33, 129 unequal}, alignments
+1 / 8 / 16, with and without weights.  The seven other logical ranks are host
+threads on the same pinned rings; what they receive from the GPU is captured
+and compared too (TX parity).
+"""
 
 from __future__ import annotations
 
@@ -10,26 +19,109 @@ from helpers import make_inputs, run_dispatch, verify_captured, verify_dispatch
 
 pytestmark = pytest.mark.gpu
 
+WORLD, EXPERTS, TOPK = 8, 256, 8
 
-def _buffer(world=8, rank=0, tmax=64, hidden=512, topk=2, experts=16, **config):
+
+def make_buffer(world=WORLD, rank=0, tmax=129, hidden=7168, topk=TOPK, experts=EXPERTS, **config):
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config.setdefault("timeout_ms", 5000)
+    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "peer_threads") if key in config}
     return HostStagedEPBuffer(num_max_tokens_per_rank=tmax, hidden=hidden, num_topk=topk, num_experts=experts,
-                              config=HostStagedConfig(**config), num_ranks=world, rank=rank)
+                              config=HostStagedConfig(**config), num_ranks=world, rank=rank, **extra)
+
+
+def check_case(buffer, label, tokens, pattern="random", expand=True, alignment=1, weights=True, seed=7, capture=True,
+               hidden=None, topk=None, experts=None, world=None, fp8=False, gaussian=False):
+    world = world or buffer.num_ranks
+    hidden, topk, experts = hidden or buffer.hidden, topk or buffer.num_topk, experts or buffer.num_experts
+    print(f"case: {label} pattern={pattern} tokens={tokens} expand={expand} alignment={alignment} weights={weights} seed={seed}", flush=True)
+    inputs = make_inputs(world, tokens, hidden, experts, topk, pattern, seed=seed, gaussian=gaussian)
+    result, _ = run_dispatch(buffer, inputs, expand=expand, alignment=alignment, zero_padding=expand, with_weights=weights, capture=capture)
+    summary = verify_dispatch(result, inputs, buffer.rank_idx, world, experts, topk, expand, alignment, expand, with_weights=weights, fp8_wire=fp8)
+    if capture:
+        verify_captured(buffer.peers, inputs, buffer.rank_idx, world, experts, topk, fp8_wire=fp8, with_weights=weights)
+    return summary
 
 
 def test_cpu_plumbing_configuration():
-    """8 logical ranks, T=64, H=512 BF16, 16 experts, top-2, softmax weights,
-    BF16 wire, expand on: layout, counts, offsets and rows against the oracle."""
-    world, tokens, hidden, experts, topk = 8, 64, 512, 16, 2
-    inputs = make_inputs(world, [tokens] * world, hidden, experts, topk, "random", seed=1, gaussian=True)
-    with _buffer(world, 0, tokens, hidden, topk, experts, channels=4) as buffer:
-        print("case: plumbing expand", flush=True)
-        result, _ = run_dispatch(buffer, inputs, expand=True, capture=True)
-        verify_dispatch(result, inputs, 0, world, experts, topk, True, 1, False)
-        assert verify_captured(buffer.peers, inputs, 0, world, experts, topk) > 0
-        del result
-        print("case: plumbing unique", flush=True)
-        result, _ = run_dispatch(buffer, inputs, expand=False, capture=True, peers_already_set=True)
-        verify_dispatch(result, inputs, 0, world, experts, topk, False, 1, False)
+    """8 logical ranks, T=64, H=512 BF16 N(0,1), 16 experts (2 per rank), top-2,
+    softmax weights, BF16 wire, expand on."""
+    with make_buffer(tmax=64, hidden=512, topk=2, experts=16, channels=4) as buffer:
+        summary = check_case(buffer, "plumbing", [64] * 8, gaussian=True, seed=1)
+        assert summary["expanded"] > 0
+        check_case(buffer, "plumbing-unique", [64] * 8, expand=False, gaussian=True, seed=1)
+
+
+@pytest.mark.parametrize("slots,descriptors", [(1, 1), (2, 3), (3, 2), (256, 256)])
+def test_ring_windows_and_patterns(slots, descriptors):
+    """Tiny rings force slot reuse, descriptor credit waits and tail drains."""
+    with make_buffer(payload_slots=slots, descriptor_slots=descriptors, channels=2, hidden=1024) as buffer:
+        for pattern in ("random", "local", "multicast", "hotspot", "partial", "none"):
+            for expand in (False, True):
+                check_case(buffer, f"Q{slots}L{descriptors}", [17] * 8, pattern, expand)
+        check_case(buffer, "empty", [0] * 8)
+        check_case(buffer, "unequal", [0] + [max(1, 129 - r * 3) for r in range(1, 8)])
+        check_case(buffer, "aligned16", [33] * 8, alignment=16)
+        for i in range(6):
+            check_case(buffer, "repeat", [3 + i % 5] * 8, expand=bool(i % 2), alignment=8, seed=100 + i)
+        check_case(buffer, "no-weights", [5] * 8, "multicast", weights=False)
+
+
+def test_full_hidden_32_channels():
+    with make_buffer(channels=32) as buffer:
+        check_case(buffer, "h7168", [129] * 8)
+        check_case(buffer, "h7168-unique", [129] * 8, expand=False, seed=9)
+        check_case(buffer, "h7168-gpu-empty", [0] + [129] * 7, seed=10)
+
+
+@pytest.mark.parametrize("rank", [3, 7])
+def test_other_local_rank(rank):
+    with make_buffer(rank=rank, channels=3, hidden=512, payload_slots=4, descriptor_slots=4) as buffer:
+        check_case(buffer, f"rank{rank}", [40] * 8)
+        check_case(buffer, f"rank{rank}-unique", [40] * 8, expand=False, alignment=1)
+
+
+@pytest.mark.parametrize("hidden", [129, 24, 8, 1])
+def test_odd_hidden_sizes(hidden):
+    """Rows that are not a multiple of 16 bytes take the scalar path."""
+    with make_buffer(hidden=hidden, channels=2, payload_slots=3, descriptor_slots=3) as buffer:
+        check_case(buffer, f"h{hidden}", [37] * 8)
+        check_case(buffer, f"h{hidden}-unique", [37] * 8, expand=False)
+
+
+def test_small_world_and_topk_shapes():
+    with make_buffer(world=2, tmax=50, hidden=256, topk=4, experts=8, channels=1, payload_slots=2, descriptor_slots=2) as buffer:
+        check_case(buffer, "p2", [50, 31])
+    with make_buffer(world=16, tmax=20, hidden=64, topk=32, experts=64, channels=5) as buffer:
+        check_case(buffer, "p16k32", [20] * 16)
+        check_case(buffer, "p16k32-unique", [20] * 16, expand=False)
+    with make_buffer(world=1, tmax=16, hidden=64, topk=2, experts=4, channels=2) as buffer:
+        check_case(buffer, "p1", [16], capture=False)
+
+
+def test_large_hidden_multi_pass():
+    """A row longer than one register pass (16 KiB) is moved in several passes."""
+    with make_buffer(hidden=12288, tmax=20, channels=2) as buffer:
+        check_case(buffer, "h12288", [20] * 8)
+
+
+def test_wave_counts():
+    for tx_waves, rx_waves in ((1, 1), (4, 6)):
+        with make_buffer(hidden=512, channels=4, payload_slots=2, descriptor_slots=2, tx_waves=tx_waves, rx_waves=rx_waves) as buffer:
+            check_case(buffer, f"tx{tx_waves}rx{rx_waves}", [60] * 8)
+
+
+def test_invalid_routes_raise_code_two():
+    """Duplicate, < -1 and >= E ids are terminal error 2 (tests/test_integration.py:222-260)."""
+    for bad in ([3, 3], [-2, 1], [256, 1]):
+        with make_buffer(hidden=64, topk=2, channels=2, timeout_ms=500) as buffer:
+            inputs = make_inputs(8, [4] * 8, 64, 256, 2, seed=3)
+            inputs[0][1][1] = torch.tensor(bad)
+            x, idx, weights = (item.cuda() for item in inputs[0])
+            result = buffer.dispatch(x, idx, weights, do_expand=True)
+            with pytest.raises(RuntimeError, match="GPU error"):
+                buffer.check_errors()
+            assert int(result[3].error[0].cpu()) == 2
+            with pytest.raises(RuntimeError, match="failed"):
+                buffer.dispatch(x, idx, weights, do_expand=True)
