@@ -1,0 +1,300 @@
+"""Benchmark of the host-staged dispatch on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens 8192] [--wire bf16|fp8] [--routing uniform|hotspot]
+
+One step is one full dispatch of the receiver's share: the GPU is logical rank
+0 of 8; its own T tokens go through the real TX path into the pinned host ring,
+the 7 other sources are pre-staged by host threads in the same rings and are
+read once over PCIe and expanded into expert-major rows in HBM.  Inputs of the
+GPU's own source are resident in HBM before the timed region; remote payloads
+are resident in pinned host memory, which is where this transport has them by
+definition.
+
+Prints ONE JSON line (metric of BASELINE.json: dispatch time and PCIe payload
+rate against the measured pinned-copy peak, T=8192, H=7168, top-8) with
+``roofline`` (stand-alone expand kernel against HBM), ``pcie`` (the transport
+kernel against the measured pinned hipMemcpy peak) and ``cpu_baseline`` (the
+reference semantics of layout+expand in PyTorch on the host cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for entry in (ROOT, ROOT / "pcie-ep_amd", ROOT / "tests"):
+    if str(entry) not in sys.path:
+        sys.path.insert(0, str(entry))
+
+WORLD, EXPERTS, HIDDEN = 8, 256, 7168
+HBM_PEAK_GBPS = 8000.0
+
+
+def log(*items) -> None:
+    print(*items, file=sys.stderr, flush=True)
+
+
+def build_inputs(tokens: int, topk: int, routing: str, heavy_tail: bool):
+    import numpy as np
+    import torch
+
+    inputs = []
+    hot = None
+    if routing == "hotspot":
+        arrays = np.load(ROOT / "tests" / "golden" / "hotspot_20_80_routes.npz", allow_pickle=False)
+        hot = (arrays["indices"], arrays["weights"])
+    for rank in range(WORLD):
+        generator = torch.Generator().manual_seed(20261024 + rank * 104729 + tokens)
+        x = torch.randn(tokens, HIDDEN, generator=generator)
+        if heavy_tail:
+            channels = torch.randperm(HIDDEN, generator=torch.Generator().manual_seed(7))[: HIDDEN // 100]
+            x[:, channels] *= 50.0
+        x = x.to(torch.bfloat16).contiguous()
+        if hot is not None:
+            idx = torch.from_numpy(hot[0][rank, :tokens].copy())
+            weights = torch.from_numpy(hot[1][rank, :tokens].copy())
+        else:
+            idx = torch.rand(tokens, EXPERTS, generator=generator).topk(topk, dim=1).indices.contiguous()
+            weights = torch.softmax(torch.randn(tokens, topk, generator=generator), dim=1).contiguous()
+        inputs.append((x, idx, weights))
+    return inputs
+
+
+def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000):
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    config = HostStagedConfig(channels=channels, stage=7 if wire == "fp8" else 6, wire_dtype="fp8_e4m3" if wire == "fp8" else "bf16",
+                              fuse_receive_expand=fuse, receive_expand_mode="pipelined" if fuse else "scalar", timeout_ms=timeout_ms)
+    return HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
+                              num_ranks=WORLD, rank=0)
+
+
+def set_peers(buffer, inputs):
+    for source in range(1, WORLD):
+        buffer.peers.set_source(source, *inputs[source])
+
+
+def cpu_baseline(inputs, payload_bytes, budget_s=20.0, fp8=False):
+    """Oracle-side layout+expand in PyTorch on the host cores (reported only)."""
+    import torch
+
+    from oracle import cpu_baseline as baseline
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    all_x, all_idx, all_w = zip(*inputs)
+    sample_tokens = all_x[0].shape[0]
+    sample = "full workload"
+    started = time.perf_counter()
+    out = baseline.layout_and_expand(all_x, all_idx, all_w, 0, EXPERTS, 1, fp8)
+    first = time.perf_counter() - started
+    if first > budget_s / 4:  # bound the CPU work: time a prefix of every source instead
+        sample_tokens = max(256, int(sample_tokens * (budget_s / 8) / first))
+        sample = f"first {sample_tokens} tokens of every source"
+        all_x, all_idx, all_w = ([t[:sample_tokens] for t in group] for group in (all_x, all_idx, all_w))
+        out = baseline.layout_and_expand(all_x, all_idx, all_w, 0, EXPERTS, 1, fp8)
+    times = []
+    deadline = time.perf_counter() + budget_s
+    for _ in range(5):
+        started = time.perf_counter()
+        out = baseline.layout_and_expand(all_x, all_idx, all_w, 0, EXPERTS, 1, fp8)
+        times.append(time.perf_counter() - started)
+        if time.perf_counter() > deadline:
+            break
+    mean = sum(times) / len(times)
+    idx0 = all_idx[0]
+    remote = (idx0 // (EXPERTS // WORLD) != 0) & (idx0 >= 0)
+    own_remote_tokens = int(remote.any(dim=1).sum())
+    moved = (own_remote_tokens + out["remote_unique"]) * payload_bytes
+    return {
+        "value": moved / mean / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port", "sample": sample,
+        "us": mean * 1e6, "min_us": min(times) * 1e6, "runs": len(times),
+        "expand_GBps": ((out["remote_unique"] + out["local_unique"]) + out["expanded_count"]) * HIDDEN * 2 / mean / 1e9,
+    }
+
+
+def measure_expand(inputs, tokens, topk, channels, repeats=20):
+    """Stand-alone expand kernel (unique rows -> expert-major rows) against HBM."""
+    import torch
+
+    from helpers import verify_dispatch
+
+    buffer = make_buffer(tokens, topk, "bf16", channels, fuse=False)
+    try:
+        set_peers(buffer, inputs)
+        buffer.peers.start(1)
+        x, idx, weights = (item.cuda() for item in inputs[0])
+        result = buffer.dispatch(x, idx, weights, do_expand=True)
+        torch.cuda.synchronize()
+        buffer.peers.wait(120_000)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, topk, True, 1, False)
+        handle = result[3]
+        unique, expanded = int(handle.unique_count.cpu()), int(handle.expanded_count.cpu())
+        pool = next(pool for pool in buffer.runtime._pools if not pool.idle())
+        plan = handle._layout
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(3):
+            buffer.runtime.expand_unique(pool.tensors, plan, 1, False)
+        torch.cuda.synchronize()
+        durations = []
+        for _ in range(repeats):
+            begin.record()
+            buffer.runtime.expand_unique(pool.tensors, plan, 1, False)
+            end.record()
+            end.synchronize()
+            durations.append(begin.elapsed_time(end))
+        mean_ms = sum(durations) / len(durations)
+        algorithmic = (unique + expanded) * HIDDEN * 2 + expanded * 36
+        del result, handle
+        return {
+            "bound": "hbm", "kernel": "expand_kernel", "achieved": algorithmic / mean_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": algorithmic / mean_ms / 1e6 / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": algorithmic,
+            "avg_us": mean_ms * 1e3, "min_us": min(durations) * 1e3, "unique_rows": unique, "expanded_rows": expanded,
+        }
+    finally:
+        buffer.close()
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--tokens", type=int, default=8192)
+    parser.add_argument("--wire", choices=("bf16", "fp8"), default="bf16")
+    parser.add_argument("--routing", choices=("uniform", "hotspot"), default="uniform")
+    parser.add_argument("--channels", type=int, default=32)
+    parser.add_argument("--skip-cpu-baseline", action="store_true")
+    parser.add_argument("--skip-expand", action="store_true")
+    parser.add_argument("--skip-verify", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's share of the dispatch; --gpus {args.gpus} is not supported "
+              "(this build uses no second GPU, no collective and no rank code)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from helpers import verify_dispatch
+    from pcie_ep import _native
+
+    torch.cuda.set_device(0)
+    topk = 4 if args.routing == "hotspot" else 8
+    tokens = args.tokens
+    log(f"[bench] building inputs: T={tokens} H={HIDDEN} top-{topk} {args.routing} {args.wire} wire")
+    inputs = build_inputs(tokens, topk, args.routing, heavy_tail=args.wire == "fp8")
+
+    h2d, d2h = _native.C.c_double(), _native.C.c_double()
+    _native.check(_native.library().pcie_ep_measure_pinned_copy(0, 1 << 30, 5, _native.C.byref(h2d), _native.C.byref(d2h)), invalid=RuntimeError)
+    log(f"[bench] pinned hipMemcpy peak: H2D {h2d.value:.2f} GB/s, D2H {d2h.value:.2f} GB/s")
+
+    buffer = make_buffer(tokens, topk, args.wire, args.channels, fuse=True)
+    sizes = buffer.runtime.sizes
+    payload_bytes, meta_bytes = int(sizes.payload_bytes), int(sizes.meta_bytes)
+    set_peers(buffer, inputs)
+    x, idx, weights = (item.cuda() for item in inputs[0])
+    total = args.warmup + args.steps + (0 if args.skip_verify else 1)
+    buffer.peers.start(total)
+    buffer.peers.wait_staged(120_000)
+    log("[bench] peers staged; warming up")
+    buffer.runtime.set_kernel_timing(True)
+    for _ in range(args.warmup):
+        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+        del result
+    torch.cuda.synchronize()
+    kernel_ms = {"prologue": [], "transport": [], "epilogue": []}
+    inside_ns = []
+    started = time.perf_counter()
+    for _ in range(args.steps):
+        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+        stamps = result[3].transport_timestamps_ns
+        # Reading the per-kernel events waits for this dispatch only; the next
+        # one is submitted right after, as a steady caller would.
+        times = buffer.runtime.kernel_times_ms()
+        for name in kernel_ms:
+            kernel_ms[name].append(times[name])
+        inside_ns.append(stamps.clone())
+        del result, stamps
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    ms_per_step = elapsed / args.steps * 1e3
+    buffer.runtime.set_kernel_timing(False)
+    inside_ns = [item.cpu().tolist() for item in inside_ns]
+
+    # One more, checked bit for bit against the oracle (untimed).
+    parity = "skipped"
+    result = None
+    if not args.skip_verify:
+        result = buffer.dispatch(x, idx, weights, do_expand=True)
+        torch.cuda.synchronize()
+    buffer.peers.wait(120_000)
+    if result is not None:
+        summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, topk, True, 1, False, fp8_wire=args.wire == "fp8")
+        parity = "bit-exact vs oracle"
+        stats = summary["stats"]
+        unique, expanded = summary["unique"], summary["expanded"]
+    else:
+        probe = buffer._last_handle
+        stats = probe.stats.cpu().tolist()
+        unique, expanded = int(probe.unique_count.cpu()), int(probe.expanded_count.cpu())
+    del result
+    own_writes, remote_reads, descriptors = int(stats[0]), int(stats[1]), int(stats[7])
+    local_unique = unique - remote_reads
+    buffer.close()
+
+    mean = lambda values: sum(values) / len(values)
+    transport_ms = mean(kernel_ms["transport"])
+    dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"]) + mean(kernel_ms["epilogue"])
+    read_bytes = remote_reads * (payload_bytes + meta_bytes + 32)
+    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 40 + remote_reads * 16
+    peak = max(h2d.value, d2h.value)
+    step_s = ms_per_step * 1e-3
+    value = (own_writes + remote_reads) * payload_bytes / step_s / 1e9
+    pcie = {
+        "bound": "pcie", "kernel": "transport_kernel", "avg_us": transport_ms * 1e3, "min_us": min(kernel_ms["transport"]) * 1e3,
+        "inside_kernel_us": mean([(end - begin) / 1e3 for begin, end in inside_ns]),
+        "read_GBps": read_bytes / (transport_ms * 1e-3) / 1e9, "write_GBps": write_bytes / (transport_ms * 1e-3) / 1e9,
+        "read_payload_GBps": remote_reads * payload_bytes / (transport_ms * 1e-3) / 1e9,
+        "peak_h2d_GBps": h2d.value, "peak_d2h_GBps": d2h.value,
+        "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d.value,
+        "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
+    }
+    record = {
+        "metric": "dispatch PCIe payload GB/s ((U+F_r)*B/t) and us per dispatch, receiver rank 0 of 8",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.wire == "bf16" else "fp8_e4m3 wire / bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"T={tokens}/source x 8 logical ranks, h{HIDDEN}, top-{topk} {args.routing}, {EXPERTS} experts (32 local), "
+                        f"{args.wire} wire, C{args.channels}, Q=L=256, expand on, own TX + 7 host-staged sources",
+            "tokens_per_rank": tokens, "hidden": HIDDEN, "topk": topk, "experts": EXPERTS, "channels": args.channels, "wire": args.wire,
+        },
+        "dispatch_us": ms_per_step * 1e3, "dispatch_gpu_us": dispatch_gpu_ms * 1e3,
+        "kernel_us": {name: mean(values) * 1e3 for name, values in kernel_ms.items()},
+        "pcie_pct_of_peak": 100.0 * pcie["frac"],
+        "logical_GBps": tokens * topk * HIDDEN * 2 / step_s / 1e9,
+        "rows": {"own_published": own_writes, "remote_unique": remote_reads, "local_unique": local_unique, "expanded": expanded},
+        "parity": parity,
+        "pcie": pcie,
+    }
+    if not args.skip_expand:
+        log("[bench] measuring the stand-alone expand kernel")
+        record["roofline"] = measure_expand(inputs, tokens, topk, args.channels)
+    else:
+        record["roofline"] = None
+    if not args.skip_cpu_baseline:
+        log("[bench] timing the CPU baseline on the host cores")
+        record["cpu_baseline"] = cpu_baseline(inputs, payload_bytes, fp8=args.wire == "fp8")
+    else:
+        record["cpu_baseline"] = None
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -98,29 +98,104 @@ __device__ inline void test_delay(uint64_t ticks) {
     while (now_ticks() - start < ticks) __builtin_amdgcn_s_sleep(16);
 }
 
-// ---- system-scope signals on pinned host memory ------------------------------
+// ---- pinned, fine-grained host memory -----------------------------------------------
+// Ordinary loads and stores to the host segments may be served from / parked in
+// the GPU's L2 and only become coherent with the CPU through the cache
+// write-back and invalidate that full system-scope release / acquire fences
+// perform.  On a kernel that is streaming hundreds of MB of expert rows into
+// HBM that write-back costs microseconds per signal.  The hot path therefore
+// gives every access to host memory the system-scope cache policy (sc0 sc1:
+// write-through, never served from a GPU cache):
+//   * payload and metadata move through buffer instructions with that policy
+//     (host_resource / host_load_* / host_store_*); out-of-range lanes are
+//     dropped by the buffer bounds check, so rows need no per-lane predicate;
+//   * signals and descriptor fields use system-scope relaxed atomics, which get
+//     the same policy;
+//   * host_store_release waits until every earlier load has returned and every
+//     earlier store has been acknowledged (the counters are wave-wide) and then
+//     stores the signal; host_load is a relaxed load whose dependants are issued
+//     after it returned.
+// The full-fence versions remain for the once-per-dispatch paths (count
+// mailbox, receive prefixes), where plain accesses are used.
+
+constexpr int kHostPolicy = 17;  // sc0 | sc1
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t host_resource(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, int(bytes), 0x00020000);
+}
+__device__ __forceinline__ u32x4 host_load_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b128(resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ void host_store_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, u32x4 value) {
+    __builtin_amdgcn_raw_buffer_store_b128(value, resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ uint32_t host_load_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b32(resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ void host_store_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint32_t value) {
+    __builtin_amdgcn_raw_buffer_store_b32(value, resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ uint16_t host_load_b16(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b16(resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ void host_store_b16(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint16_t value) {
+    __builtin_amdgcn_raw_buffer_store_b16(value, resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ uint8_t host_load_b8(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b8(resource, int(byte_offset), 0, kHostPolicy);
+}
+__device__ __forceinline__ void host_store_b8(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint8_t value) {
+    __builtin_amdgcn_raw_buffer_store_b8(value, resource, int(byte_offset), 0, kHostPolicy);
+}
+template <typename T>
+__device__ __forceinline__ T host_field_load(const T* address) {
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+template <typename T>
+__device__ __forceinline__ void host_field_store(T* address, T value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__device__ __forceinline__ void wait_memory_ops() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void compiler_barrier() { asm volatile("" ::: "memory"); }
+
+__device__ __forceinline__ uint64_t host_load(const uint64_t* address) {
+    const uint64_t value = __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    compiler_barrier();
+    return value;
+}
+__device__ __forceinline__ void host_store_release(uint64_t* address, uint64_t value) {
+    wait_memory_ops();
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 __device__ __forceinline__ uint64_t load_acquire_system(const uint64_t* address) {
     return __hip_atomic_load(address, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
-}
-__device__ __forceinline__ uint64_t load_relaxed_system(const uint64_t* address) {
-    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 __device__ __forceinline__ void store_release_system(uint64_t* address, uint64_t value) {
     __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 __device__ __forceinline__ void fence_acquire_system() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
-__device__ __forceinline__ void fence_release_system() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
 
 // ---- workgroup-scope hand-off through LDS -----------------------------------
+// Role wavefronts of one workgroup exchange tickets and counters through LDS.
+// The fences are restricted to the LDS address space: a wavefront that has
+// megabytes of global loads/stores in flight must not drain them just to bump
+// a counter.  Global data handed over together with a ticket is made visible
+// explicitly by its writer (wait_memory_ops) and read with device-scope loads.
 
+__device__ __forceinline__ void fence_lds() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup", "local"); }
 __device__ __forceinline__ int lds_load(const int* address) {
-    return __hip_atomic_load(address, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    const int value = __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return value;
 }
 __device__ __forceinline__ void lds_store(int* address, int value) {
-    __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-__device__ __forceinline__ void fence_workgroup() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); }
+__device__ __forceinline__ int device_load(const int* address) {
+    return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // ---- device-scope flags in HBM -----------------------------------------------
 

@@ -217,7 +217,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint16_t* x, uint8_
     const int waves_per_block = blockDim.x / kWave;
     const int total_waves = gridDim.x * waves_per_block;
     for (int token = blockIdx.x * waves_per_block + threadIdx.x / kWave; token < tokens; token += total_waves) {
-        const float scale = quantize_row<kVector>(x + size_t(token) * hidden, codes + size_t(token) * hidden, hidden, lane);
+        const float scale = quantize_row<kVector>(x + size_t(token) * hidden, DeviceCodes{codes + size_t(token) * hidden}, hidden, lane);
         if (lane == 0) scales[token] = scale;
     }
 }

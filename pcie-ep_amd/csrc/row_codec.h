@@ -30,9 +30,42 @@ __device__ inline void copy_row(const uint16_t* input, uint16_t* output, int hid
     }
 }
 
-// Returns the row scale.  kVector requires hidden % 16 == 0.
+// Where a quantised row goes: device memory, or a host slot through buffer
+// stores with the system-scope cache policy.
+struct DeviceCodes {
+    uint8_t* output;
+    __device__ __forceinline__ void vector(int group, u32x4 codes) const { reinterpret_cast<u32x4*>(output)[group] = codes; }
+    __device__ __forceinline__ void single(int index, uint8_t code) const { output[index] = code; }
+};
+struct HostCodes {
+    __amdgpu_buffer_rsrc_t slot;
+    __device__ __forceinline__ void vector(int group, u32x4 codes) const { host_store_b128(slot, uint32_t(group) * 16u, codes); }
+    __device__ __forceinline__ void single(int index, uint8_t code) const { host_store_b8(slot, uint32_t(index), code); }
+};
+
+// BF16 row from device memory into a host slot.
 template <bool kVector>
-__device__ inline float quantize_row(const uint16_t* input, uint8_t* output, int hidden, int lane) {
+__device__ inline void copy_row_to_host(const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int hidden, int lane) {
+    if constexpr (kVector) {
+        const int vectors = hidden / 8;
+        const u32x4* source = reinterpret_cast<const u32x4*>(input);
+        for (int first = 0; first < vectors; first += kPassItems * kWave) {
+            RowVectors row;
+            row_load_vectors<true>(row, source, first, vectors, lane);
+#pragma unroll
+            for (int j = 0; j < kPassItems; ++j) {
+                const int index = first + j * kWave + lane;
+                if (index < vectors) host_store_b128(slot, uint32_t(index) * 16u, row.v[j]);
+            }
+        }
+    } else {
+        for (int index = lane; index < hidden; index += kWave) host_store_b16(slot, uint32_t(index) * 2u, input[index]);
+    }
+}
+
+// Returns the row scale.  kVector requires hidden % 16 == 0.
+template <bool kVector, typename Sink>
+__device__ inline float quantize_row(const uint16_t* input, const Sink& sink, int hidden, int lane) {
     // Sweep 1: row amax in FP32.  Sweep 2 re-reads the row (it is L2 resident).
     float amax = 0.0f;
     if constexpr (kVector) {
@@ -58,7 +91,6 @@ __device__ inline float quantize_row(const uint16_t* input, uint8_t* output, int
         // 16 elements (two 16-byte loads) -> 16 codes (one 16-byte store) per lane.
         const int groups = hidden / 16;
         const u32x4* source = reinterpret_cast<const u32x4*>(input);
-        u32x4* destination = reinterpret_cast<u32x4*>(output);
         for (int group = lane; group < groups; group += kWave) {
             const u32x4 lo = source[group * 2], hi = source[group * 2 + 1];
             u32x4 codes;
@@ -71,10 +103,10 @@ __device__ inline float quantize_row(const uint16_t* input, uint8_t* output, int
                               uint32_t(fp8_quantize_element(uint16_t(b & 0xFFFFu), inverse)) << 16 |
                               uint32_t(fp8_quantize_element(uint16_t(b >> 16), inverse)) << 24;
             }
-            destination[group] = codes;
+            sink.vector(group, codes);
         }
     } else {
-        for (int index = lane; index < hidden; index += kWave) output[index] = fp8_quantize_element(input[index], inverse);
+        for (int index = lane; index < hidden; index += kWave) sink.single(index, fp8_quantize_element(input[index], inverse));
     }
     return scale;
 }

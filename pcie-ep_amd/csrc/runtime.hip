@@ -105,6 +105,11 @@ struct pcie_ep_runtime {
     int counts_ack_skip_source = -1;
     std::unique_ptr<PeerEmulator> peers;
     bool closed = false;
+    // Optional per-kernel timing with HIP events on the launch stream.
+    bool timing = false;
+    bool timing_valid = false;
+    int timing_kernels = 0;
+    hipEvent_t marks[5] = {};
 };
 
 namespace {
@@ -294,6 +299,8 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     }
     if (rt->epoch) (void)hipFree(rt->epoch);
     if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
+    for (hipEvent_t mark : rt->marks)
+        if (mark) (void)hipEventDestroy(mark);
     delete rt;
     return status;
 }
@@ -308,10 +315,42 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     //   transport = the channel kernel (TX, RX, receive prefixes, fused expand)
     //   epilogue  = copy_local_tokens + zero_padding + reduce_statistics
     // and the separate expand when receive/expand fusion is off.
+    const bool timed = rt->timing;
+    rt->timing_valid = false;
+    if (timed) HIP_TRY(hipEventRecord(rt->marks[0], stream));
     HIP_TRY(launch_prologue(state, stream));
+    if (timed) HIP_TRY(hipEventRecord(rt->marks[1], stream));
     HIP_TRY(launch_transport(state, stream));
+    if (timed) HIP_TRY(hipEventRecord(rt->marks[2], stream));
     HIP_TRY(launch_epilogue(state, stream));
-    if (state.expand && !state.fuse_expand) HIP_TRY(launch_expand(state, stream));
+    if (timed) HIP_TRY(hipEventRecord(rt->marks[3], stream));
+    const bool separate_expand = state.expand && !state.fuse_expand;
+    if (separate_expand) HIP_TRY(launch_expand(state, stream));
+    if (timed) {
+        HIP_TRY(hipEventRecord(rt->marks[4], stream));
+        rt->timing_kernels = separate_expand ? 4 : 3;
+        rt->timing_valid = true;
+    }
+    return 0;
+}
+
+int pcie_ep_set_kernel_timing(pcie_ep_runtime* rt, int32_t enable) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (enable && !rt->marks[0])
+        for (hipEvent_t& mark : rt->marks) HIP_TRY(hipEventCreate(&mark));
+    rt->timing = enable != 0;
+    rt->timing_valid = false;
+    return 0;
+}
+
+int pcie_ep_get_kernel_times(pcie_ep_runtime* rt, float* milliseconds) {
+    if (!rt || rt->closed || !milliseconds) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!rt->timing_valid) return set_error(PCIE_EP_E_STATE, "no timed dispatch has been recorded");
+    HIP_TRY(hipEventSynchronize(rt->marks[4]));
+    for (int kernel = 0; kernel < 4; ++kernel) {
+        milliseconds[kernel] = 0.0f;
+        if (kernel < rt->timing_kernels) HIP_TRY(hipEventElapsedTime(milliseconds + kernel, rt->marks[kernel], rt->marks[kernel + 1]));
+    }
     return 0;
 }
 

@@ -59,7 +59,8 @@ struct Queues {
     int rx_total;
     int pad;
     int tx_done[kMaxTxWaves];  // tickets completed by each TX worker
-    int rx_done[kMaxRxWaves];
+    int rx_done[kMaxRxWaves];     // tickets whose ring entry an RX worker has copied out
+    int rx_retired[kMaxRxWaves];  // tickets an RX worker has finished (row read, ACK sent, stores issued)
     TxTicket tx[kTxRing];
     RxTicket rx[kRxRing];
     uint32_t scratch[kMaxTxWaves + kMaxRxWaves][kScratchDwords];
@@ -265,8 +266,7 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
             const uint64_t still = __ballot(pending);
             const int first_pending = still ? __builtin_ctzll(still) : kWave;
             const int head = produced + __popcll(batch & lanes_below(first_pending));
-            __threadfence();  // ring history + ticket bodies before the head
-            fence_workgroup();
+            wait_memory_ops();  // ring history (global) and ticket bodies (LDS) before the head
             if (lane == 0) lds_store(&q.tx_head, head);
             if (!still) break;
             ++stage_busy;
@@ -305,10 +305,10 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
             const int destination = lane % ranks;
             bool acked = true;
             if (lane < per_pass * ranks && my_ordinal < produced) {
-                const int token = state.chan_remote_tokens[size_t(channel) * stride + my_ordinal];
+                const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
                 const uint32_t remote = state.plan_mask[token] & ~(1u << me);
                 if ((remote >> destination) & 1u)
-                    acked = load_acquire_system(ack_at(z, own, channel, my_ordinal % slots, destination)) == sequence(epoch, token);
+                    acked = host_load(ack_at(z, own, channel, my_ordinal % slots, destination)) == sequence(epoch, token);
             }
             const uint64_t missing = __ballot(!acked);
             if (!missing) drain_ordinal += per_pass;
@@ -373,7 +373,7 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
         const bool want = member && ordinal < expected;
         Descriptor* descriptor = descriptor_at(z, state.seg[member ? source : me], channel, me, want ? ordinal : 0);
         bool ready = false;
-        if (want) ready = load_acquire_system(&descriptor->ready) == sequence(epoch, ordinal);
+        if (want) ready = host_load(&descriptor->ready) == sequence(epoch, ordinal);
         const uint64_t ready_lanes = __ballot(ready);
         // Descriptors of one source are consumed in order: accept the leading run.
         const uint64_t group = (ready_lanes >> (source < ranks ? source * lookahead : 0)) & group_mask;
@@ -389,9 +389,9 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
         int slot = 0, token = 0;
         uint64_t payload_sequence = 0;
         if (accept) {
-            slot = descriptor->payload_slot;
-            token = descriptor->token_index;
-            payload_sequence = descriptor->payload_sequence;
+            slot = host_field_load(&descriptor->payload_slot);
+            token = host_field_load(&descriptor->token_index);
+            payload_sequence = host_field_load(&descriptor->payload_sequence);
         }
         bool pending = accept;
         while (true) {
@@ -404,13 +404,13 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
                 ticket.payload_sequence = payload_sequence;
                 // The descriptor is captured: return its credit.  The payload ACK
                 // and the local ticket slot are separate resources.
-                store_release_system(&descriptor->consumed, sequence(epoch, ordinal));
+                host_store_release(&descriptor->consumed, sequence(epoch, ordinal));
                 pending = false;
             }
             const uint64_t still = __ballot(pending);
             const int first_pending = still ? __builtin_ctzll(still) : kWave;
             const int head = issued + __popcll(accepted & lanes_below(first_pending));
-            fence_workgroup();
+            fence_lds();
             if (lane == 0) lds_store(&q.rx_head, head);
             if (!still) break;
             if (broadcast_first(lds_load(&q.abort))) {
@@ -425,7 +425,7 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
     // RX is finished when every worker has retired its tickets.
     while (true) {
         if (broadcast_first(lds_load(&q.abort))) break;
-        int done = lane < state.rx_waves ? lds_load(q.rx_done + lane) : 0;
+        int done = lane < state.rx_waves ? lds_load(q.rx_retired + lane) : 0;
         for (int offset = 32; offset > 0; offset >>= 1) done += __shfl_xor(done, offset);
         if (done >= issued && issued >= total) break;
         backoff();
@@ -441,12 +441,11 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
 // TX payload worker
 // ---------------------------------------------------------------------------------------
 template <bool kFp8, bool kVector>
-__device__ void tx_copy_row(const DeviceState& state, const uint16_t* input, char* slot, uint32_t* scratch, int lane) {
+__device__ float tx_copy_row(const DeviceState& state, const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int lane) {
     const int hidden = state.z.dims.hidden;
-    float scale = 1.0f;
-    if constexpr (kFp8) scale = quantize_row<kVector>(input, reinterpret_cast<uint8_t*>(slot), hidden, lane);
-    else copy_row<kVector, false>(input, reinterpret_cast<uint16_t*>(slot), hidden, lane);
-    if (lane == 0) scratch[2] = float_bits(scale);
+    if constexpr (kFp8) return quantize_row<kVector>(input, HostCodes{slot}, hidden, lane);
+    copy_row_to_host<kVector>(input, slot, hidden, lane);
+    return 1.0f;
 }
 
 template <bool kFp8, bool kVector>
@@ -462,8 +461,7 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
     int64_t writes = 0, deliveries = 0, credit_miss = 0;
     for (int ticket_index = worker;; ticket_index += state.tx_waves) {
         if (wait_ticket(q, &q.tx_head, &q.tx_total, ticket_index, lane) < 0) break;
-        fence_workgroup();
-        __threadfence();
+        fence_lds();
         const TxTicket& ticket = q.tx[ticket_index % kTxRing];
         const int token = ticket.token, ordinal = ticket.ordinal;
         const uint32_t endpoints = ticket.endpoints;
@@ -478,7 +476,7 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
         bool slot_ok = true, credit_ok = true;
         uint64_t previous_sequence = 0;
         if (ordinal >= slots) {
-            const int previous_token = state.chan_remote_tokens[size_t(channel) * stride + ordinal - slots];
+            const int previous_token = device_load(state.chan_remote_tokens + size_t(channel) * stride + ordinal - slots);
             const uint32_t previous_remote = state.plan_mask[previous_token] & ~(1u << me);
             slot_ok = !(lane < ranks && ((previous_remote >> lane) & 1u));
             previous_sequence = sequence(epoch, previous_token);
@@ -486,9 +484,9 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
         if (targeted && my_descriptor >= descriptors) credit_ok = false;
         bool aborted = false;
         while (true) {
-            if (!slot_ok) slot_ok = load_acquire_system(ack_at(z, own, channel, slot, lane)) == previous_sequence;
+            if (!slot_ok) slot_ok = host_load(ack_at(z, own, channel, slot, lane)) == previous_sequence;
             if (!credit_ok)
-                credit_ok = load_acquire_system(&descriptor_at(z, own, channel, lane, my_descriptor)->consumed) ==
+                credit_ok = host_load(&descriptor_at(z, own, channel, lane, my_descriptor)->consumed) ==
                             sequence(epoch, my_descriptor - descriptors);
             if (__all(slot_ok && credit_ok)) break;
             ++credit_miss;
@@ -499,13 +497,13 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
             backoff();
         }
         if (aborted) break;
-        fence_acquire_system();
+        compiler_barrier();
 
         // Slot metadata: composed in this wavefront's LDS scratch, then copied out
         // as consecutive dwords.  Weights are the live ones of this dispatch.
         char* slot_base = slot_at(z, own, channel, slot);
         for (int index = lane; index < meta_dwords; index += kWave) scratch[index] = 0;
-        fence_workgroup();
+        fence_lds();
         if (lane == 0) {
             scratch[0] = uint32_t(token);
             scratch[1] = state.plan_mask[token];
@@ -518,26 +516,28 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
                 float_bits(state.topk_weights ? state.topk_weights[size_t(token) * topk + lane] : 1.0f);
         }
         if (lane == kWave - 1) test_delay(state.tx_delay);
-        tx_copy_row<kFp8, kVector>(state, state.x + size_t(token) * z.dims.hidden, slot_base, scratch, lane);
-        fence_workgroup();
+        const __amdgpu_buffer_rsrc_t slot_resource = host_resource(slot_base, uint32_t(z.meta_offset + z.meta_bytes));
+        const float scale = tx_copy_row<kFp8, kVector>(state, state.x + size_t(token) * z.dims.hidden,
+                                                       host_resource(slot_base, uint32_t(z.payload_bytes)), lane);
+        if (lane == 0) scratch[2] = float_bits(scale);
+        fence_lds();
         if (lane == meta_dwords - 1 || (lane == kWave - 1 && meta_dwords > kWave)) test_delay(state.metadata_delay);
-        uint32_t* meta = reinterpret_cast<uint32_t*>(slot_base + z.meta_offset);
-        for (int index = lane; index < meta_dwords; index += kWave) meta[index] = scratch[index];
-        // Every lane's payload and metadata stores are complete at system scope
-        // before any lane publishes a descriptor.
-        __threadfence_system();
+        for (int index = lane; index < meta_dwords; index += kWave)
+            host_store_b32(slot_resource, uint32_t(z.meta_offset + index * 4), scratch[index]);
+        // Every lane's payload and metadata stores have been acknowledged before
+        // any lane publishes a descriptor (the counters are wave-wide).
+        wait_memory_ops();
         if (targeted) {
             Descriptor* descriptor = descriptor_at(z, own, channel, lane, my_descriptor);
-            descriptor->payload_sequence = sequence(epoch, token);
-            descriptor->payload_slot = slot;
-            descriptor->token_index = token;
-            descriptor->rank_ordinal = int32_t(scratch[kMetaRankOrdinalsOffset / 4 + lane]);
-            store_release_system(&descriptor->ready, sequence(epoch, my_descriptor));
+            host_field_store(&descriptor->payload_sequence, sequence(epoch, token));
+            host_field_store(&descriptor->payload_slot, int32_t(slot));
+            host_field_store(&descriptor->token_index, int32_t(token));
+            host_field_store(&descriptor->rank_ordinal, int32_t(scratch[kMetaRankOrdinalsOffset / 4 + lane]));
+            host_store_release(&descriptor->ready, sequence(epoch, my_descriptor));
         }
         if (ticket_index == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
         ++writes;
         deliveries += __popc(endpoints);
-        fence_workgroup();
         if (lane == 0) lds_store(q.tx_done + worker, ticket_index / state.tx_waves + 1);
     }
     if (lane == 0) {
@@ -564,23 +564,25 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
     const int hidden = z.dims.hidden;
     const uint64_t epoch = *state.epoch;
     uint32_t* scratch = q.scratch[kMaxTxWaves + worker];
-    const int meta_dwords = z.meta_bytes / 4;
     const bool scatter = state.expand && state.fuse_expand;
     int64_t reads = 0;
     for (int ticket_index = worker;; ticket_index += state.rx_waves) {
         if (wait_ticket(q, &q.rx_head, &q.rx_total, ticket_index, lane) < 0) break;
-        fence_workgroup();
-        fence_acquire_system();
+        fence_lds();
         const RxTicket ticket = q.rx[ticket_index % kRxRing];
+        // The ticket now lives in registers: its ring entry may be reused while
+        // this wavefront is still moving the row.
+        fence_lds();
+        if (lane == 0) lds_store(q.rx_done + worker, ticket_index / state.rx_waves + 1);
         const int source = ticket.source;
         const char* slot_base = slot_at(z, state.seg[source], channel, ticket.slot);
+        const __amdgpu_buffer_rsrc_t payload = host_resource(slot_base, uint32_t(z.payload_bytes));
+        const __amdgpu_buffer_rsrc_t slot_meta = host_resource(slot_base + z.meta_offset, uint32_t(z.meta_bytes));
         if (lane == kWave - 1) test_delay(state.rx_delay);
 
         // Metadata first (it arrives first), payload right behind it.
-        const uint32_t* meta = reinterpret_cast<const uint32_t*>(slot_base + z.meta_offset);
-        uint32_t meta_lo = 0, meta_hi = 0;
-        if (lane < meta_dwords) meta_lo = __builtin_nontemporal_load(meta + lane);
-        if (kWave + lane < meta_dwords) meta_hi = __builtin_nontemporal_load(meta + kWave + lane);
+        const uint32_t meta_lo = host_load_b32(slot_meta, uint32_t(lane) * 4u);  // out of range reads as 0
+        const uint32_t meta_hi = host_load_b32(slot_meta, uint32_t(kWave + lane) * 4u);
 
         RowVectors row;
         const int wire_vectors = kFp8 ? hidden / 16 : hidden / 8;
@@ -591,15 +593,16 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
 #pragma unroll
                 for (int j = 0; j < kPassItems / 2; ++j) {
                     const int index = j * kWave + lane;
-                    row.v[j] = index < wire_vectors ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(slot_base) + index) : u32x4{0u, 0u, 0u, 0u};
+                    row.v[j] = host_load_b128(payload, uint32_t(index) * 16u);
                 }
             } else {
-                row_load_vectors<true>(row, reinterpret_cast<const u32x4*>(slot_base), 0, wire_vectors, lane);
+#pragma unroll
+                for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(j * kWave + lane) * 16u);
             }
         }
         scratch[lane] = meta_lo;
         if (kWave + lane < kScratchDwords) scratch[kWave + lane] = meta_hi;
-        fence_workgroup();
+        fence_lds();
         const int token = int(scratch[0]);
         const float scale = bits_float(scratch[2]);
         bool bad = token != ticket.token || ticket.payload_sequence != sequence(epoch, token);
@@ -648,17 +651,18 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
 #pragma unroll
                         for (int j = 0; j < kPassItems / 2; ++j) {
                             const int index = first_wire + j * kWave + lane;
-                            row.v[j] = index < wire_vectors ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(slot_base) + index) : u32x4{0u, 0u, 0u, 0u};
+                            row.v[j] = host_load_b128(payload, uint32_t(index) * 16u);
                         }
                     } else {
-                        row_load_vectors<true>(row, reinterpret_cast<const u32x4*>(slot_base), first_wire, wire_vectors, lane);
+#pragma unroll
+                        for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(first_wire + j * kWave + lane) * 16u);
                     }
                 }
                 const bool last_pass = first_wire + wire_per_pass >= wire_vectors;
                 if (last_pass) {
                     // All loads of the staged row have returned: release the host
                     // slot.  The release orders them before the ACK store.
-                    if (lane == 0) store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
                 }
                 if constexpr (kFp8) {
                     // 16 codes -> 16 BF16 (two 16-byte vectors); expanded in place from the top.
@@ -699,12 +703,12 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                 for (int j = 0; j < kPassScalars; ++j) {
                     const int index = first + j * kWave + lane;
                     if (index < hidden) {
-                        if constexpr (kFp8) items.v[j] = fp8_dequantize_element(reinterpret_cast<const uint8_t*>(slot_base)[index], scale);
-                        else items.v[j] = reinterpret_cast<const uint16_t*>(slot_base)[index];
+                        if constexpr (kFp8) items.v[j] = fp8_dequantize_element(host_load_b8(payload, uint32_t(index)), scale);
+                        else items.v[j] = host_load_b16(payload, uint32_t(index) * 2u);
                     }
                 }
                 if (first + kPassScalars * kWave >= hidden) {
-                    if (lane == 0) store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
                 }
                 uint64_t remaining = destinations;
                 while (remaining) {
@@ -720,7 +724,7 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                 }
             }
             if (hidden == 0 && lane == 0)
-                store_release_system(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
         }
 
         // Row metadata (advanced_layout.cuh:207-215; layout.cuh:31-48).
@@ -748,9 +752,7 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
             }
         }
         ++reads;
-        __threadfence();
-        fence_workgroup();
-        if (lane == 0) lds_store(q.rx_done + worker, ticket_index / state.rx_waves + 1);
+        if (lane == 0) lds_store(q.rx_retired + worker, ticket_index / state.rx_waves + 1);
     }
     if (lane == 0)
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatHostReads),
@@ -771,7 +773,7 @@ __global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
         q.tx_total = -1;
         q.rx_total = -1;
         for (int i = 0; i < kMaxTxWaves; ++i) q.tx_done[i] = 0;
-        for (int i = 0; i < kMaxRxWaves; ++i) q.rx_done[i] = 0;
+        for (int i = 0; i < kMaxRxWaves; ++i) q.rx_done[i] = q.rx_retired[i] = 0;
     }
     // One immutable entry verdict for the whole workgroup: branching on the
     // mutable abort flag here could strand a wavefront at the final barrier

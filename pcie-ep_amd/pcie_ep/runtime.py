@@ -227,6 +227,15 @@ class NativeRuntime:
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _native.check(self._lib.pcie_ep_expand_unique(self._require(), C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
 
+    def set_kernel_timing(self, enable: bool) -> None:
+        _native.check(self._lib.pcie_ep_set_kernel_timing(self._require(), int(enable)), invalid=RuntimeError)
+
+    def kernel_times_ms(self) -> Dict[str, float]:
+        """Durations of the last timed dispatch's kernels (waits for it to finish)."""
+        values = (C.c_float * 4)()
+        _native.check(self._lib.pcie_ep_get_kernel_times(self._require(), values), invalid=RuntimeError)
+        return dict(zip(("prologue", "transport", "epilogue", "expand"), (float(v) for v in values)))
+
     def pool_tensors(self, index: int) -> Dict[str, torch.Tensor]:
         return self._pools[index].tensors
 

@@ -195,3 +195,37 @@ def test_channel_counts_sum_to_rank_counts():
     assert channel.sum(axis=0).tolist() == layout.counts[:P].tolist()
     remote = layout.remote_tokens(2)
     assert np.all(np.diff(remote) > 0)
+
+
+@pytest.mark.parametrize("alignment,fp8", [(1, False), (8, False), (4, True)])
+def test_cpu_baseline_matches_oracle(alignment, fp8):
+    """The torch implementation that bench.py times as the CPU baseline produces
+    exactly the oracle's layout and rows."""
+    from oracle import cpu_baseline, fp8_oracle
+
+    rng = np.random.default_rng(2)
+    ranks, experts, topk, hidden = 4, 32, 3, 48
+    sizes = [9, 0, 14, 6]
+    all_idx = [_random_routes(rng, t, topk, experts, partial=True) for t in sizes]
+    generator = torch.Generator().manual_seed(4)
+    all_x = [torch.randn(t, hidden, generator=generator).to(torch.bfloat16) for t in sizes]
+    all_w = [torch.rand(t, topk, generator=generator) for t in sizes]
+    for rank in range(ranks):
+        expectation = oracle.expected_dispatch(all_idx, rank, ranks, experts, alignment)
+        out = cpu_baseline.layout_and_expand(all_x, [torch.from_numpy(i) for i in all_idx], all_w, rank, experts, alignment, fp8)
+        receiver, e = expectation.receiver, expectation.expanded
+        assert out["expert_counts"].tolist() == receiver.expert_counts.tolist()
+        assert out["expert_offsets"].tolist() == receiver.expert_offsets.tolist()
+        assert out["expert_prefix"].tolist() == receiver.expert_prefix.tolist()
+        assert out["source_offsets"].tolist() == receiver.source_offsets.tolist()
+        assert (out["unique_count"], out["expanded_count"]) == (receiver.unique_count, receiver.expanded_count)
+        assert np.array_equal(out["source_meta"].numpy()[e.rows], np.stack([e.source, e.token, e.branch], axis=1))
+        assert np.array_equal(out["recv_idx"].numpy()[e.rows], e.expert)
+        for i, row in enumerate(e.rows):
+            source, token, branch = int(e.source[i]), int(e.token[i]), int(e.branch[i])
+            want = all_x[source][token : token + 1]
+            if fp8 and source != rank:
+                want = fp8_oracle.roundtrip(want)
+            assert torch.equal(out["recv_x"][row].view(torch.int16), want[0].view(torch.int16))
+            assert out["recv_weights"][row] == all_w[source][token, branch]
+        assert not torch.count_nonzero(out["recv_x"][torch.from_numpy(e.padding_rows)].view(torch.int16))
