@@ -49,12 +49,14 @@ typedef struct pcie_ep_config {
     int32_t wire_fp8;           /* 0 BF16 wire, 1 E4M3FN + FP32 scale per token */
     int32_t timeout_ms;         /* device-side protocol timeout */
     int32_t fuse_receive_expand;/* 1: receive waves scatter to expert rows; 0: unique rows + expand kernel */
-    int32_t tx_waves;           /* payload TX wavefronts per channel, 0 = default */
-    int32_t rx_waves;           /* payload RX wavefronts per channel, 0 = default */
+    int32_t tx_waves;           /* payload TX wavefronts per payload workgroup, 0 = default (1) */
+    int32_t rx_waves;           /* payload RX wavefronts per payload workgroup, 0 = default (2) */
     int32_t peer_threads;       /* host threads standing in for the other ranks; 0 = none */
     int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
     int32_t device;             /* HIP device ordinal */
-    int32_t reserved[7];
+    int32_t worker_groups;      /* payload workgroups of the transport kernel, spread over the XCDs;
+                                   0 = default (48), -1 = none (control workgroups move the rows) */
+    int32_t reserved[6];
 } pcie_ep_config;
 
 /* Capacities and byte sizes a caller needs to allocate pools
@@ -70,7 +72,8 @@ typedef struct pcie_ep_sizes {
     int32_t meta_bytes;         /* per-slot token metadata bytes */
     int32_t mailbox_dwords;
     int32_t transport_threads;  /* workgroup size of the transport kernel */
-    int32_t reserved[7];
+    int32_t transport_workgroups;
+    int32_t reserved[6];
 } pcie_ep_sizes;
 
 /* One dispatch: inputs, the route plan to fill or reuse, and every output of

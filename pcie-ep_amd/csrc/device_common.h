@@ -16,6 +16,52 @@ constexpr uint64_t kPrefixFailed = ~uint64_t(0);
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// Work queues of the transport kernel, in device memory.  Control wavefronts
+// (one TX and one RX control per channel) produce tickets into two global
+// rings; payload wavefronts of ANY workgroup, and therefore of any XCD, claim
+// them.  A row is thus moved by whichever wavefront is free: channels are load
+// balanced against each other, every channel is served by all eight XCDs (the
+// XCDs get unequal shares of the host link), and the number of rows in flight
+// - which sets the latency every control-path read sees - is chosen by the
+// number of worker wavefronts, not by the number of channels.
+// All fields are accessed with device-scope (cross-XCD coherent) operations;
+// the per-entry tags carry the epoch, so the rings need no clearing.
+constexpr int kRing = 2048;
+
+struct alignas(16) RxEntry {
+    int32_t source;
+    int32_t slot;
+    int32_t token;
+    int32_t channel;
+    uint64_t payload_sequence;
+    uint64_t reserved;
+};
+struct alignas(16) TxEntry {
+    int32_t token;
+    int32_t ordinal;  // position among this channel's remote tokens
+    uint32_t endpoints;
+    int32_t channel;
+    int32_t descriptor_ordinal[kMaxRanks];
+};
+static_assert(sizeof(RxEntry) == 32 && sizeof(TxEntry) == 80, "queue entry layout");
+
+struct alignas(128) QueueCounter {
+    uint32_t value;
+    int32_t total;  // -1 until the number of tickets is known
+    char pad[120];
+};
+
+struct alignas(256) TransportQueues {
+    QueueCounter rx_tail, tx_tail;  // tickets reserved by producers (fetch-add)
+    QueueCounter rx_head, tx_head;  // tickets claimed by workers (fetch-add); .total = tickets of this dispatch
+    QueueCounter abort;             // value != 0: every role exits
+    QueueCounter rx_retired[kMaxChannels], tx_retired[kMaxChannels], rx_finished[kMaxChannels];
+    uint64_t rx_ready[kRing], rx_taken[kRing];  // sequence(epoch, n): entry n % kRing holds / has been copied out
+    uint64_t tx_ready[kRing], tx_taken[kRing];
+    RxEntry rx[kRing];
+    TxEntry tx[kRing];
+};
+
 // Launch argument of every kernel: this rank's device pointers, the device
 // aliases of the pinned host segments and the plan/output pool of one dispatch
 // (the role of AdvancedDeviceState: csrc/kernels/host_staged/advanced_common.cuh:86-129).
@@ -23,8 +69,6 @@ struct DeviceState {
     SegmentLayout z;
     char* seg[kMaxRanks];
     int local_rank;
-    int tx_waves;
-    int rx_waves;
     int fuse_expand;  // receive waves scatter straight into expert rows
     int expand;
     int alignment;
@@ -49,6 +93,9 @@ struct DeviceState {
     int32_t* plan_chan_remote;// [C]
 
     int32_t* chan_remote_tokens;  // scratch [C, ceil(Tmax / C)]: ring history for slot reuse
+    TransportQueues* queues;
+    int worker_groups;            // payload workgroups after the C control workgroups (spread over the XCDs)
+    int tx_waves, rx_waves;       // payload wavefronts per payload workgroup
 
     uint16_t* unique_payload;
     int64_t* unique_topk_idx;
@@ -193,8 +240,29 @@ __device__ __forceinline__ void lds_store(int* address, int value) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-__device__ __forceinline__ int device_load(const int* address) {
+// Device-scope (cross-XCD coherent) accesses.  As with host memory, data that
+// crosses workgroups is always accessed with the coherent cache policy and
+// ordered with wait_memory_ops(), never with cache write-back fences.
+constexpr int kDevicePolicy = 16;  // sc1
+template <typename T>
+__device__ __forceinline__ T device_load(const T* address) {
     return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ void device_store(T* address, T value) {
+    __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t device_add(uint32_t* address, uint32_t value) {
+    return __hip_atomic_fetch_add(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_resource(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, int(bytes), 0x00020000);
+}
+__device__ __forceinline__ uint32_t device_load_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b32(resource, int(byte_offset), 0, kDevicePolicy);
+}
+__device__ __forceinline__ void device_store_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint32_t value) {
+    __builtin_amdgcn_raw_buffer_store_b32(value, resource, int(byte_offset), 0, kDevicePolicy);
 }
 
 // ---- device-scope flags in HBM -----------------------------------------------

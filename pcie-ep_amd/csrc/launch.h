@@ -7,16 +7,22 @@
 
 namespace pcie_ep {
 
-constexpr int kDefaultTxWaves = 2;
-constexpr int kDefaultRxWaves = 4;
+// Payload workgroups of the transport kernel (after the C control workgroups)
+// and the TX / RX payload wavefronts each of them carries.  The defaults keep
+// about 1.4 MB of host reads in flight: enough to saturate a Gen5 x16 link,
+// little enough that control-path reads are not queued behind them for long.
+constexpr int kDefaultWorkerGroups = 48;
+constexpr int kDefaultTxWaves = 1;
+constexpr int kDefaultRxWaves = 2;
 constexpr int kMaxTxWaves = 4;
 constexpr int kMaxRxWaves = 6;
+constexpr int kMaxWorkerGroups = 1024;
 
 // Epoch begin + layout + count publication (one workgroup).
 hipError_t launch_prologue(const DeviceState& state, hipStream_t stream);
 // Channel transport: control / TX / RX-scatter wavefront roles, one workgroup per channel.
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream);
-int transport_threads(int tx_waves, int rx_waves);
+int transport_threads(const DeviceState& state);
 // Local bypass copy, alignment-gap zeroing and statistics reduction.
 hipError_t launch_epilogue(const DeviceState& state, hipStream_t stream);
 // Stand-alone expand of unique rows into expert-major rows (+ padding).

@@ -67,6 +67,20 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
         state.receive_prefix_state[i] = 0;
     }
     for (int i = threadIdx.x; i < (channels + 1) * 2; i += blockDim.x) state.prefix_tx_timestamps_ns[i] = 0;
+    // Ticket queues of the transport kernel: counters back to zero, totals
+    // unknown.  The rings' tags carry the epoch and need no clearing.
+    {
+        TransportQueues& q = *state.queues;
+        QueueCounter* globals[] = {&q.rx_tail, &q.tx_tail, &q.rx_head, &q.tx_head, &q.abort};
+        if (threadIdx.x < 5) {
+            globals[threadIdx.x]->value = 0;
+            globals[threadIdx.x]->total = -1;
+        }
+        for (int i = threadIdx.x; i < channels; i += blockDim.x) {
+            q.rx_retired[i].value = q.tx_retired[i].value = q.rx_finished[i].value = 0;
+            q.rx_retired[i].total = q.tx_retired[i].total = q.rx_finished[i].total = -1;
+        }
+    }
 
     // Abort signals are terminal.  Issue the loads now; the verdict is taken
     // after the layout so their PCIe latency hides behind it.
@@ -218,6 +232,12 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
     }
     __syncthreads();
     if (mailbox_failed) return;
+    // Transmit tickets of this dispatch: every own token with a remote destination.
+    if (threadIdx.x == 0) {
+        int remote_tokens = 0;
+        for (int channel = 0; channel < channels; ++channel) remote_tokens += state.plan_chan_remote[channel];
+        state.queues->tx_head.total = remote_tokens;
+    }
     publish_counts(state, epoch);
 }
 

@@ -85,6 +85,8 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
         return set_error(PCIE_EP_E_INVALID, "invalid advanced capacity or timeout");
     if (c->tx_waves < 0 || c->tx_waves > kMaxTxWaves || c->rx_waves < 0 || c->rx_waves > kMaxRxWaves)
         return set_error(PCIE_EP_E_INVALID, "tx_waves must be 0..%d and rx_waves 0..%d", kMaxTxWaves, kMaxRxWaves);
+    if (c->worker_groups < -1 || c->worker_groups > kMaxWorkerGroups)
+        return set_error(PCIE_EP_E_INVALID, "worker_groups must be -1..%d", kMaxWorkerGroups);
     if (c->peer_threads < 0) return set_error(PCIE_EP_E_INVALID, "peer_threads must be non-negative");
     dims = Dimensions{c->num_ranks, c->max_tokens, c->hidden, c->topk, c->num_experts, c->channels, c->payload_slots, c->descriptor_slots,
                       c->wire_fp8 ? 1 : 0};
@@ -100,7 +102,8 @@ struct pcie_ep_runtime {
     char* segments[kMaxRanks] = {};
     uint64_t* epoch = nullptr;
     int32_t* chan_remote_tokens = nullptr;
-    int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves;
+    int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves, worker_groups = kDefaultWorkerGroups;
+    TransportQueues* queues = nullptr;
     uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
     int counts_ack_skip_source = -1;
     std::unique_ptr<PeerEmulator> peers;
@@ -140,6 +143,8 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.z = rt->z;
     for (int rank = 0; rank < d.num_ranks; ++rank) s.seg[rank] = rt->segments[rank];
     s.local_rank = rt->config.local_rank;
+    s.queues = rt->queues;
+    s.worker_groups = rt->worker_groups;
     s.tx_waves = rt->tx_waves;
     s.rx_waves = rt->rx_waves;
     s.fuse_expand = rt->config.fuse_receive_expand ? 1 : 0;
@@ -221,8 +226,12 @@ int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes) {
     sizes->payload_bytes = z.payload_bytes;
     sizes->meta_bytes = z.meta_bytes;
     sizes->mailbox_dwords = z.mailbox_dwords;
-    sizes->transport_threads = transport_threads(config->tx_waves ? config->tx_waves : kDefaultTxWaves,
-                                                 config->rx_waves ? config->rx_waves : kDefaultRxWaves);
+    DeviceState probe{};
+    probe.tx_waves = config->tx_waves ? config->tx_waves : kDefaultTxWaves;
+    probe.rx_waves = config->rx_waves ? config->rx_waves : kDefaultRxWaves;
+    probe.worker_groups = config->worker_groups < 0 ? 0 : (config->worker_groups ? config->worker_groups : kDefaultWorkerGroups);
+    sizes->transport_threads = transport_threads(probe);
+    sizes->transport_workgroups = config->channels + probe.worker_groups;
     return 0;
 }
 
@@ -241,6 +250,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     rt->plan = plan_layout(dims);
     if (config->tx_waves) rt->tx_waves = config->tx_waves;
     if (config->rx_waves) rt->rx_waves = config->rx_waves;
+    if (config->worker_groups) rt->worker_groups = config->worker_groups < 0 ? 0 : config->worker_groups;
 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers
     // /dev/shm mappings: advanced_shared_memory.hpp:264-288).  First touch is
@@ -272,6 +282,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (error == hipSuccess) error = hipMemset(rt->epoch, 0, 256);
         if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->chan_remote_tokens), history);
         if (error == hipSuccess) error = hipMemset(rt->chan_remote_tokens, 0, history);
+        if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->queues), sizeof(TransportQueues));
+        if (error == hipSuccess) error = hipMemset(rt->queues, 0, sizeof(TransportQueues));
         if (error == hipSuccess) error = hipDeviceSynchronize();
         if (error != hipSuccess) status = set_error(PCIE_EP_E_HIP, "device workspace allocation failed: %s", hipGetErrorString(error));
     }
@@ -280,6 +292,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
             if (segment) (void)hipHostFree(segment);
         if (rt->epoch) (void)hipFree(rt->epoch);
         if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
+        if (rt->queues) (void)hipFree(rt->queues);
         return status;
     }
     if (config->peer_threads > 0 && dims.num_ranks > 1)
@@ -299,6 +312,7 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     }
     if (rt->epoch) (void)hipFree(rt->epoch);
     if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
+    if (rt->queues) (void)hipFree(rt->queues);
     for (hipEvent_t mark : rt->marks)
         if (mark) (void)hipEventDestroy(mark);
     delete rt;

@@ -1,6 +1,6 @@
-// Channel transport kernel: one workgroup per channel, wavefronts specialised
-// into TX control (+ guardian), RX control (+ receive prefixes), TX payload
-// workers and RX/scatter workers.
+// Channel transport kernel: TX control (+ guardian), RX control (+ receive
+// prefixes), TX payload workers and RX/scatter workers, all as single
+// wavefronts with their own role.
 //
 // Replaces advanced_transport_pipelined and its roles
 // (csrc/kernels/host_staged/fused_receive.cuh:333-360;
@@ -8,19 +8,29 @@
 // tx_worker; fused_receive.cuh:199-305 producer/consumer) and, for the unique
 // layout, advanced_transport (advanced_dispatch.cuh:919-958).
 //
-// Differences that come from designing for 64-lane wavefronts:
+// Design for MI355X (64-lane wavefronts, 8 XCDs):
 //  * A payload worker is ONE wavefront that owns a whole row: 14 x 16-byte
 //    loads per lane are issued back to back (896 vectors of a 14 336-byte BF16
 //    row), the row lives in registers, and the same wavefront stores it to
-//    every destination expert row.  The staged row is read once, there is no
+//    every destination expert row.  The staged row is read once; there is no
 //    LDS tile and no producer/consumer hand-off (the reference stages through
 //    shared memory with 3+3 warps per ticket).
 //  * Control wavefronts work on 64 candidates at a time with ballots: TX control
 //    derives ring slots and per-destination descriptor ordinals for 64 tokens
 //    from popcounts of ballots; RX control probes up to 64/P descriptors per
 //    source per iteration instead of one source per iteration.
-//  * Workers publish their own descriptors and payload ACKs as soon as their
-//    own fence has completed; control wavefronts only reserve and hand out work.
+//  * Work is handed out through two global ticket rings in device memory (one
+//    for TX, one for RX).  Workgroup b < C is the control workgroup of channel
+//    b (TX control + RX control); the workgroups after them only hold payload
+//    wavefronts, which claim tickets of ANY channel.  Consecutive workgroup ids
+//    land on consecutive XCDs, so every channel's rows are moved by all eight
+//    XCDs.  This matters because the XCDs get unequal shares of the host link:
+//    with workers bound to their channel's workgroup, equal work finished in
+//    8.8 ms on the best XCD and 12.8 ms on the worst.  It also decouples the
+//    bytes in flight (worker wavefronts x row size), which set the latency of
+//    every control-path read, from the number of channels.
+//  * Workers publish their own descriptors and payload ACKs as soon as their own
+//    stores / loads have completed; control wavefronts only reserve and hand out.
 #include "device_common.h"
 #include "launch.h"
 #include "row_codec.h"
@@ -29,59 +39,58 @@ namespace pcie_ep {
 
 namespace {
 
-constexpr int kTxRing = 32;
-constexpr int kRxRing = 32;
-constexpr int kScratchDwords = 128;  // per worker wavefront: one slot metadata record
+constexpr int kScratchDwords = 128;  // per wavefront: one slot metadata record or one ticket
+constexpr int kMaxWaves = 12;
 
-struct TxTicket {
-    int token;
-    int ordinal;  // position among this channel's remote tokens
-    uint32_t endpoints;
-    int pad;
-    int descriptor_ordinal[kMaxRanks];
+struct WaveScratch {
+    uint32_t words[kMaxWaves][kScratchDwords];
 };
 
-struct RxTicket {
-    int source;
-    int slot;
-    int token;
-    int descriptor_ordinal;
-    uint64_t payload_sequence;
+// Local time only: payload workers never scan the host abort flags themselves
+// (hundreds of wavefronts doing so would be PCIe traffic of their own); the
+// channel's guardian does and raises the channel's abort word.
+struct Deadline {
+    uint64_t start;
+    __device__ explicit Deadline(uint64_t begin) : start(begin) {}
+    __device__ bool expired(const DeviceState& state) const { return now_ticks() - start > state.timeout_ticks; }
 };
 
-struct Queues {
-    int abort;
-    int tx_finished;
-    int rx_finished;
-    int tx_head;   // tickets published by TX control
-    int tx_total;  // -1 until every ticket is published
-    int rx_head;
-    int rx_total;
-    int pad;
-    int tx_done[kMaxTxWaves];  // tickets completed by each TX worker
-    int rx_done[kMaxRxWaves];     // tickets whose ring entry an RX worker has copied out
-    int rx_retired[kMaxRxWaves];  // tickets an RX worker has finished (row read, ACK sent, stores issued)
-    TxTicket tx[kTxRing];
-    RxTicket rx[kRxRing];
-    uint32_t scratch[kMaxTxWaves + kMaxRxWaves][kScratchDwords];
-};
+__device__ __forceinline__ bool aborted(TransportQueues& q) { return device_load(&q.abort.value) != 0; }
+__device__ __forceinline__ void raise_abort(TransportQueues& q) { device_store(&q.abort.value, 1u); }
 
-__device__ __forceinline__ bool ticket_slot_free(const int* done, int workers, int ring, int ticket) {
-    const int previous = ticket - ring;
-    if (previous < 0) return true;
-    return lds_load(done + previous % workers) > previous / workers;
+// Producer side: reserve `count` consecutive tickets (one fetch-add per wavefront).
+__device__ __forceinline__ int reserve_tickets(QueueCounter& tail, int count, int lane) {
+    uint32_t base = 0;
+    if (lane == 0) base = device_add(&tail.value, uint32_t(count));
+    return broadcast_first(int(base));
+}
+__device__ __forceinline__ bool ring_entry_free(const uint64_t* taken, uint64_t epoch, int ticket) {
+    const int previous = ticket - kRing;
+    return previous < 0 || device_load(taken + previous % kRing) == sequence(epoch, previous);
 }
 
-// Wait until ticket `ticket` is published.  Returns 1 when available, -1 to exit.
-__device__ inline int wait_ticket(Queues& q, const int* head, const int* total, int ticket, int lane) {
+// Consumer side: claim the next ticket, then wait until its entry is complete.
+// Returns 1 when available, -1 when there is no such ticket or on abort.
+__device__ __forceinline__ int claim_ticket(QueueCounter& head, int lane) {
+    uint32_t ticket = 0;
+    if (lane == 0) ticket = device_add(&head.value, 1u);
+    return broadcast_first(int(ticket));
+}
+__device__ inline int wait_ticket(const DeviceState& state, TransportQueues& q, const uint64_t* ready, QueueCounter& head, int ticket,
+                                  uint64_t epoch, int lane, const Deadline& deadline) {
     while (true) {
         int action = 0;
         if (lane == 0) {
-            if (lds_load(&q.abort)) action = -1;
-            else if (lds_load(head) > ticket) action = 1;
+            if (aborted(q)) action = -1;
+            else if (device_load(ready + ticket % kRing) == sequence(epoch, ticket)) action = 1;
             else {
-                const int limit = lds_load(total);
+                const int limit = device_load(&head.total);
                 if (limit >= 0 && ticket >= limit) action = -1;
+                else if (deadline.expired(state)) {
+                    record_error(state, kErrRingProgressWait);
+                    raise_abort(q);
+                    action = -1;
+                }
             }
         }
         action = broadcast_first(action);
@@ -167,9 +176,12 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         const int channel = index / ranks, source = index % ranks;
         state.expected_receive_counts[index] = mailbox_at(z, state.seg[source], me)[1 + local + channel];
     }
+    const int own_unique = __shfl(unique, me);
     if (lane == 0) {
         *state.unique_count = total_unique;
         *state.expanded_count = expanded_total;
+        // Receive tickets of this dispatch: every unique row of a remote source.
+        device_store(&state.queues->rx_head.total, total_unique - own_unique);
     }
     // ACK a source only after every lane captured its counts: the source may
     // overwrite the mailbox for the next epoch afterwards (advanced_layout.cuh:91-93).
@@ -212,7 +224,7 @@ __device__ bool prepare_receive_prefixes(const DeviceState& state, int lane) {
 // ---------------------------------------------------------------------------------------
 // TX control + guardian
 // ---------------------------------------------------------------------------------------
-__device__ void tx_control(const DeviceState& state, Queues& q, int channel, int lane) {
+__device__ void tx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, channels = z.dims.channels, me = state.local_rank;
     const int slots = z.dims.payload_slots;
@@ -225,6 +237,7 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;
     const uint64_t below = lanes_below(lane);
+    const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
     int produced = 0;
     int reserved[kMaxRanks];
 #pragma unroll
@@ -250,27 +263,27 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
             }
         }
         // Ring history: which token occupied ordinal i (needed when a slot is reused).
-        if (remote) state.chan_remote_tokens[size_t(channel) * stride + ordinal] = token;
+        if (remote) device_store(state.chan_remote_tokens + size_t(channel) * stride + ordinal, token);
+        const int ticket_index = reserve_tickets(q.tx_tail, __popcll(batch), lane) + __popcll(batch & below);
         bool pending = remote != 0;
         while (true) {
-            if (pending && ticket_slot_free(q.tx_done, state.tx_waves, kTxRing, ordinal)) {
-                TxTicket& ticket = q.tx[ordinal % kTxRing];
-                ticket.token = token;
-                ticket.ordinal = ordinal;
-                ticket.endpoints = remote;
+            if (pending && ring_entry_free(q.tx_taken, epoch, ticket_index)) {
+                const uint32_t at = uint32_t(ticket_index % kRing) * uint32_t(sizeof(TxEntry));
+                device_store_b32(ring, at + 0, uint32_t(token));
+                device_store_b32(ring, at + 4, uint32_t(ordinal));
+                device_store_b32(ring, at + 8, remote);
+                device_store_b32(ring, at + 12, uint32_t(channel));
 #pragma unroll
                 for (int rank = 0; rank < kMaxRanks; ++rank)
-                    if (rank < ranks) ticket.descriptor_ordinal[rank] = my_descriptor[rank];
+                    if (rank < ranks) device_store_b32(ring, at + 16 + 4 * rank, uint32_t(my_descriptor[rank]));
+                // Ring history and the ticket body are complete before the tag.
+                wait_memory_ops();
+                device_store(q.tx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
                 pending = false;
             }
-            const uint64_t still = __ballot(pending);
-            const int first_pending = still ? __builtin_ctzll(still) : kWave;
-            const int head = produced + __popcll(batch & lanes_below(first_pending));
-            wait_memory_ops();  // ring history (global) and ticket bodies (LDS) before the head
-            if (lane == 0) lds_store(&q.tx_head, head);
-            if (!still) break;
+            if (!__any(pending)) break;
             ++stage_busy;
-            if (health.poll(state, lane) || broadcast_first(lds_load(&q.abort))) {
+            if (health.poll(state, lane) || broadcast_first(aborted(q) ? 1 : 0)) {
                 failed = true;
                 break;
             }
@@ -278,26 +291,16 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
         }
         produced += __popcll(batch);
     }
-    if (lane == 0) lds_store(&q.tx_total, produced);
 
     // Wait for the workers, then drain the ACKs of the last ring window: earlier
     // slots were checked when they were reused (advanced_dispatch.cuh:229-285).
     // Lanes poll different (ordinal, destination) pairs in parallel.
     bool drained = failed;
     int drain_ordinal = produced > slots ? produced - slots : 0;
-    bool workers_finished = false;
+    bool workers_finished = false, announced = false;
     while (true) {
-        int verdict = 0;
-        if (lane == 0) {
-            if (lds_load(&q.abort)) verdict = -1;
-        }
-        verdict = broadcast_first(verdict);
-        if (verdict < 0) break;
-        if (!workers_finished) {
-            int done = lane < state.tx_waves ? lds_load(q.tx_done + lane) : 0;
-            for (int offset = 32; offset > 0; offset >>= 1) done += __shfl_xor(done, offset);
-            workers_finished = done >= produced;
-        }
+        if (broadcast_first(aborted(q) ? 1 : 0)) break;
+        if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
         if (workers_finished && !drained) {
             // Each pass checks up to 64 / P ordinals with one lane per destination.
             const int per_pass = kWave / ranks;
@@ -316,8 +319,13 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
             if (drain_ordinal >= produced) drained = true;
         }
         if (workers_finished && drained) {
-            if (lane == 0 && !lds_load(&q.tx_finished)) lds_store(&q.tx_finished, 1);
-            if (broadcast_first(lds_load(&q.rx_finished))) break;
+            if (!announced) {
+                // Diagnostic: when this channel's transmit side was drained,
+                // relative to the channel's start (column 1; column 0 is RX).
+                if (lane == 0) state.receive_expand_overlap[channel * 2 + 1] = ticks_to_ns(now_ticks() - start);
+                announced = true;
+            }
+            if (broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
         }
         // Guardian: this wavefront outlives TX so that a stalled RX still times out.
         const bool unhealthy = health.poll(state, lane);
@@ -325,32 +333,33 @@ __device__ void tx_control(const DeviceState& state, Queues& q, int channel, int
         if (unhealthy || broadcast_first(forced ? 1 : 0)) {
             if (lane == 0) {
                 record_error(state, kErrRingProgressWait);
-                lds_store(&q.abort, 1);
+                raise_abort(q);
             }
             break;
         }
         backoff();
     }
     if (lane == 0) {
-        lds_store(&q.tx_finished, 1);
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatTxStageBusy),
                   static_cast<unsigned long long>(stage_busy));
         // Only this wavefront writes the channel's mapped abort word.
-        if (lds_load(&q.abort)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
+        if (aborted(q)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
+        // Both directions are complete (or aborted): the channel's end time.
+        state.channel_timestamps_ns[channel * 2 + 1] = ticks_to_ns(now_ticks());
     }
 }
 
 // ---------------------------------------------------------------------------------------
 // RX control
 // ---------------------------------------------------------------------------------------
-__device__ void rx_control(const DeviceState& state, Queues& q, int channel, int lane) {
+__device__ void rx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, me = state.local_rank;
+    const uint64_t begin = now_ticks();
     if (!prepare_receive_prefixes(state, lane)) {
         if (lane == 0) {
-            lds_store(&q.abort, 1);
-            lds_store(&q.rx_total, 0);
-            lds_store(&q.rx_finished, 1);
+            raise_abort(q);
+            device_store(&q.rx_finished[channel].value, 1u);
         }
         return;
     }
@@ -361,14 +370,16 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
     const int expected = member ? state.expected_receive_counts[channel * ranks + source] : 0;
     int total = ahead == 0 ? expected : 0;
     for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
-    if (lane == 0) lds_store(&q.rx_total, total);
     const uint64_t below = lanes_below(lane);
-    const uint64_t group_mask = lookahead >= 64 ? ~0ull : ((1ull << lookahead) - 1ull);
+    const uint64_t group_mask = (1ull << lookahead) - 1ull;
+    const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
+    Deadline deadline(begin);
     int consumed = 0, issued = 0;
-    int64_t not_ready = 0;
+    int64_t not_ready = 0, iterations = 0, ring_waits = 0;
     bool failed = false;
     while (issued < total && !failed) {
-        if (broadcast_first(lds_load(&q.abort))) break;
+        ++iterations;
+        if (broadcast_first(aborted(q) ? 1 : 0)) break;
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
         Descriptor* descriptor = descriptor_at(z, state.seg[member ? source : me], channel, me, want ? ordinal : 0);
@@ -385,7 +396,7 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
             backoff();
             continue;
         }
-        const int ticket_index = issued + __popcll(accepted & below);
+        const int ticket_index = reserve_tickets(q.rx_tail, __popcll(accepted), lane) + __popcll(accepted & below);
         int slot = 0, token = 0;
         uint64_t payload_sequence = 0;
         if (accept) {
@@ -395,25 +406,24 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
         }
         bool pending = accept;
         while (true) {
-            if (pending && ticket_slot_free(q.rx_done, state.rx_waves, kRxRing, ticket_index)) {
-                RxTicket& ticket = q.rx[ticket_index % kRxRing];
-                ticket.source = source;
-                ticket.slot = slot;
-                ticket.token = token;
-                ticket.descriptor_ordinal = ordinal;
-                ticket.payload_sequence = payload_sequence;
-                // The descriptor is captured: return its credit.  The payload ACK
-                // and the local ticket slot are separate resources.
+            if (pending && ring_entry_free(q.rx_taken, epoch, ticket_index)) {
+                const uint32_t at = uint32_t(ticket_index % kRing) * uint32_t(sizeof(RxEntry));
+                device_store_b32(ring, at + 0, uint32_t(source));
+                device_store_b32(ring, at + 4, uint32_t(slot));
+                device_store_b32(ring, at + 8, uint32_t(token));
+                device_store_b32(ring, at + 12, uint32_t(channel));
+                device_store_b32(ring, at + 16, uint32_t(payload_sequence));
+                device_store_b32(ring, at + 20, uint32_t(payload_sequence >> 32));
+                // The descriptor is captured: return its credit (this also waits
+                // for the ticket body), then tag the entry complete.  The payload
+                // ACK and the ring entry are separate resources.
                 host_store_release(&descriptor->consumed, sequence(epoch, ordinal));
+                device_store(q.rx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
                 pending = false;
             }
-            const uint64_t still = __ballot(pending);
-            const int first_pending = still ? __builtin_ctzll(still) : kWave;
-            const int head = issued + __popcll(accepted & lanes_below(first_pending));
-            fence_lds();
-            if (lane == 0) lds_store(&q.rx_head, head);
-            if (!still) break;
-            if (broadcast_first(lds_load(&q.abort))) {
+            if (!__any(pending)) break;
+            ++ring_waits;
+            if (broadcast_first((aborted(q) || deadline.expired(state)) ? 1 : 0)) {
                 failed = true;
                 break;
             }
@@ -422,18 +432,21 @@ __device__ void rx_control(const DeviceState& state, Queues& q, int channel, int
         issued += __popcll(accepted);
         if (member) consumed += run;
     }
-    // RX is finished when every worker has retired its tickets.
+    // RX is finished when every ticket has been retired by a worker.
     while (true) {
-        if (broadcast_first(lds_load(&q.abort))) break;
-        int done = lane < state.rx_waves ? lds_load(q.rx_retired + lane) : 0;
-        for (int offset = 32; offset > 0; offset >>= 1) done += __shfl_xor(done, offset);
-        if (done >= issued && issued >= total) break;
+        if (broadcast_first(aborted(q) ? 1 : 0)) break;
+        if (broadcast_first(int(device_load(&q.rx_retired[channel].value))) >= issued && issued >= total) break;
         backoff();
     }
     if (lane == 0) {
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxNotReady),
                   static_cast<unsigned long long>(not_ready));
-        lds_store(&q.rx_finished, 1);
+        // Diagnostic: when this channel's receive side finished, relative to the
+        // channel's start (column 0), next to the transmit side's drain (column 1).
+        state.receive_expand_overlap[channel * 2] = ticks_to_ns(now_ticks() - begin);
+        state.channel_stats[channel * kStatFields + kStatMetaOverlap] = iterations;
+        state.channel_stats[channel * kStatFields + kStatTxCreditMiss] = ring_waits;
+        device_store(&q.rx_finished[channel].value, 1u);
     }
 }
 
@@ -449,26 +462,32 @@ __device__ float tx_copy_row(const DeviceState& state, const uint16_t* input, __
 }
 
 template <bool kFp8, bool kVector>
-__device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int worker, int lane) {
+__device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
     const int slots = z.dims.payload_slots, descriptors = z.dims.descriptor_slots;
     const int stride = (z.dims.max_tokens + z.dims.channels - 1) / z.dims.channels;
     char* own = state.seg[me];
     const uint64_t epoch = *state.epoch;
-    uint32_t* scratch = q.scratch[worker];
     const int meta_dwords = z.meta_bytes / 4;
+    const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
+    Deadline deadline(now_ticks());
     int64_t writes = 0, deliveries = 0, credit_miss = 0;
-    for (int ticket_index = worker;; ticket_index += state.tx_waves) {
-        if (wait_ticket(q, &q.tx_head, &q.tx_total, ticket_index, lane) < 0) break;
-        fence_lds();
-        const TxTicket& ticket = q.tx[ticket_index % kTxRing];
-        const int token = ticket.token, ordinal = ticket.ordinal;
-        const uint32_t endpoints = ticket.endpoints;
+    while (true) {
+        const int ticket_index = claim_ticket(q.tx_head, lane);
+        if (wait_ticket(state, q, q.tx_ready, q.tx_head, ticket_index, epoch, lane, deadline) < 0) break;
+        // Copy the ticket out of the ring (one dword per lane), then free its entry.
+        const uint32_t entry_base = uint32_t(ticket_index % kRing) * uint32_t(sizeof(TxEntry));
+        const uint32_t word = device_load_b32(ring, entry_base + uint32_t(lane < int(sizeof(TxEntry) / 4) ? lane : 0) * 4u);
+        const int token = __shfl(int(word), 0), ordinal = __shfl(int(word), 1);
+        const uint32_t endpoints = uint32_t(__shfl(int(word), 2));
+        const int channel = __shfl(int(word), 3);
+        const int my_descriptor = __shfl(int(word), 4 + (lane < ranks ? lane : 0));
+        wait_memory_ops();
+        if (lane == 0) device_store(q.tx_taken + ticket_index % kRing, sequence(epoch, ticket_index));
         const int slot = ordinal % slots;
-        const int my_descriptor = lane < ranks ? ticket.descriptor_ordinal[lane] : 0;
         const bool targeted = lane < ranks && ((endpoints >> lane) & 1u);
-        if (ticket_index == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(now_ticks());
+        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(now_ticks());
 
         // Flow control: the slot's previous occupant must be ACKed by all its
         // targets and a descriptor entry must have been consumed before reuse
@@ -482,7 +501,7 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
             previous_sequence = sequence(epoch, previous_token);
         }
         if (targeted && my_descriptor >= descriptors) credit_ok = false;
-        bool aborted = false;
+        bool stop = false;
         while (true) {
             if (!slot_ok) slot_ok = host_load(ack_at(z, own, channel, slot, lane)) == previous_sequence;
             if (!credit_ok)
@@ -490,13 +509,13 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
                             sequence(epoch, my_descriptor - descriptors);
             if (__all(slot_ok && credit_ok)) break;
             ++credit_miss;
-            if (broadcast_first(lds_load(&q.abort))) {
-                aborted = true;
+            if (broadcast_first((aborted(q) || deadline.expired(state)) ? 1 : 0)) {
+                stop = true;
                 break;
             }
             backoff();
         }
-        if (aborted) break;
+        if (stop) break;
         compiler_barrier();
 
         // Slot metadata: composed in this wavefront's LDS scratch, then copied out
@@ -535,13 +554,16 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
             host_field_store(&descriptor->rank_ordinal, int32_t(scratch[kMetaRankOrdinalsOffset / 4 + lane]));
             host_store_release(&descriptor->ready, sequence(epoch, my_descriptor));
         }
-        if (ticket_index == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
+        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
         ++writes;
         deliveries += __popc(endpoints);
-        if (lane == 0) lds_store(q.tx_done + worker, ticket_index / state.tx_waves + 1);
+        fence_lds();  // scratch is reused by the next ticket
+        if (lane == 0) device_add(&q.tx_retired[channel].value, 1u);
     }
-    if (lane == 0) {
-        auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields);
+    // Workers serve every channel; their counts go to channel 0's row of the
+    // per-channel statistics, whose column sums are what callers read.
+    if (lane == 0 && (writes || credit_miss)) {
+        auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats);
         atomicAdd(stats + kStatHostWrites, static_cast<unsigned long long>(writes));
         atomicAdd(stats + kStatDeliveries, static_cast<unsigned long long>(deliveries));
         atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(deliveries));
@@ -552,30 +574,29 @@ __device__ void tx_worker(const DeviceState& state, Queues& q, int channel, int 
 // ---------------------------------------------------------------------------------------
 // RX + scatter worker
 // ---------------------------------------------------------------------------------------
-struct Destinations {
-    int count;
-    int64_t row[kMaxTopk];
-};
-
 template <bool kFp8, bool kVector>
-__device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int worker, int lane) {
+__device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
     const uint64_t epoch = *state.epoch;
-    uint32_t* scratch = q.scratch[kMaxTxWaves + worker];
     const bool scatter = state.expand && state.fuse_expand;
+    const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
+    Deadline deadline(now_ticks());
     int64_t reads = 0;
-    for (int ticket_index = worker;; ticket_index += state.rx_waves) {
-        if (wait_ticket(q, &q.rx_head, &q.rx_total, ticket_index, lane) < 0) break;
-        fence_lds();
-        const RxTicket ticket = q.rx[ticket_index % kRxRing];
+    while (true) {
+        const int ticket_index = claim_ticket(q.rx_head, lane);
+        if (wait_ticket(state, q, q.rx_ready, q.rx_head, ticket_index, epoch, lane, deadline) < 0) break;
+        const uint32_t entry_base = uint32_t(ticket_index % kRing) * uint32_t(sizeof(RxEntry));
+        const uint32_t word = device_load_b32(ring, entry_base + uint32_t(lane < 8 ? lane : 0) * 4u);
+        const int source = __shfl(int(word), 0), slot = __shfl(int(word), 1), ticket_token = __shfl(int(word), 2);
+        const int channel = __shfl(int(word), 3);
+        const uint64_t payload_sequence = uint64_t(uint32_t(__shfl(int(word), 4))) | uint64_t(uint32_t(__shfl(int(word), 5))) << 32;
         // The ticket now lives in registers: its ring entry may be reused while
         // this wavefront is still moving the row.
-        fence_lds();
-        if (lane == 0) lds_store(q.rx_done + worker, ticket_index / state.rx_waves + 1);
-        const int source = ticket.source;
-        const char* slot_base = slot_at(z, state.seg[source], channel, ticket.slot);
+        wait_memory_ops();
+        if (lane == 0) device_store(q.rx_taken + ticket_index % kRing, sequence(epoch, ticket_index));
+        const char* slot_base = slot_at(z, state.seg[source], channel, slot);
         const __amdgpu_buffer_rsrc_t payload = host_resource(slot_base, uint32_t(z.payload_bytes));
         const __amdgpu_buffer_rsrc_t slot_meta = host_resource(slot_base + z.meta_offset, uint32_t(z.meta_bytes));
         if (lane == kWave - 1) test_delay(state.rx_delay);
@@ -591,27 +612,23 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
             // First (usually only) pass of the row.
             if constexpr (kFp8) {
 #pragma unroll
-                for (int j = 0; j < kPassItems / 2; ++j) {
-                    const int index = j * kWave + lane;
-                    row.v[j] = host_load_b128(payload, uint32_t(index) * 16u);
-                }
+                for (int j = 0; j < kPassItems / 2; ++j) row.v[j] = host_load_b128(payload, uint32_t(j * kWave + lane) * 16u);
             } else {
 #pragma unroll
                 for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(j * kWave + lane) * 16u);
             }
         }
         scratch[lane] = meta_lo;
-        if (kWave + lane < kScratchDwords) scratch[kWave + lane] = meta_hi;
+        scratch[kWave + lane] = meta_hi;
         fence_lds();
         const int token = int(scratch[0]);
         const float scale = bits_float(scratch[2]);
-        bool bad = token != ticket.token || ticket.payload_sequence != sequence(epoch, token);
-        if (bad) {
+        if (token != ticket_token || payload_sequence != sequence(epoch, token)) {
             // Terminal: never forge an ACK for a slot whose identity is unknown
             // (advanced_dispatch.cuh:607-610).
             if (lane == 0) {
                 record_error(state, kErrPayloadSequence);
-                lds_store(&q.abort, 1);
+                raise_abort(q);
             }
             break;
         }
@@ -621,21 +638,22 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
         int my_expert = -1;
         if (scatter) {
             if (lane < topk) {
-                const int expert = int(scratch[kMetaBranchOffset / 4 + lane]) - me * local;
-                if (int(scratch[kMetaBranchOffset / 4 + lane]) >= 0 && expert >= 0 && expert < local) {
+                const int global_expert = int(scratch[kMetaBranchOffset / 4 + lane]);
+                const int expert = global_expert - me * local;
+                if (global_expert >= 0 && expert >= 0 && expert < local) {
                     my_expert = expert;
-                    my_row = int64_t(state.expert_offsets[expert]) + state.source_expert_prefix[source * local + expert] +
+                    my_row = int64_t(device_load(state.expert_offsets + expert)) + device_load(state.source_expert_prefix + source * local + expert) +
                              int(scratch[kMetaBranchOffset / 4 + topk + lane]);
                 }
             }
         } else if (lane == 0) {
-            my_row = int64_t(state.source_offsets[source]) + int(scratch[kMetaRankOrdinalsOffset / 4 + me]);
+            my_row = int64_t(device_load(state.source_offsets + source)) + int(scratch[kMetaRankOrdinalsOffset / 4 + me]);
         }
         const int64_t capacity = scatter ? state.expanded_capacity : unique_capacity(z.dims);
         if (__any(my_row >= capacity)) {
             if (lane == 0) {
                 record_error(state, kErrExpandedCapacity);
-                lds_store(&q.abort, 1);
+                raise_abort(q);
             }
             break;
         }
@@ -649,10 +667,7 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                 if (first_wire > 0) {
                     if constexpr (kFp8) {
 #pragma unroll
-                        for (int j = 0; j < kPassItems / 2; ++j) {
-                            const int index = first_wire + j * kWave + lane;
-                            row.v[j] = host_load_b128(payload, uint32_t(index) * 16u);
-                        }
+                        for (int j = 0; j < kPassItems / 2; ++j) row.v[j] = host_load_b128(payload, uint32_t(first_wire + j * kWave + lane) * 16u);
                     } else {
 #pragma unroll
                         for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(first_wire + j * kWave + lane) * 16u);
@@ -660,9 +675,8 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                 }
                 const bool last_pass = first_wire + wire_per_pass >= wire_vectors;
                 if (last_pass) {
-                    // All loads of the staged row have returned: release the host
-                    // slot.  The release orders them before the ACK store.
-                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                    // All loads of the staged row have returned: release the host slot.
+                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, slot, me), payload_sequence);
                 }
                 if constexpr (kFp8) {
                     // 16 codes -> 16 BF16 (two 16-byte vectors); expanded in place from the top.
@@ -681,7 +695,7 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                     const int64_t out_row = __shfl(my_row, branch);
                     u32x4* output = reinterpret_cast<u32x4*>(output_base + size_t(out_row) * hidden);
                     if constexpr (kFp8) {
-                        // Lane's wire vector j*64+lane holds elements [16*i, 16*i+16) -> output vectors 2*i, 2*i+1.
+                        // Wire vector i holds elements [16 i, 16 i + 16) -> output vectors 2 i and 2 i + 1.
 #pragma unroll
                         for (int j = 0; j < kPassItems / 2; ++j) {
                             const int index = first_wire + j * kWave + lane;
@@ -708,7 +722,7 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                     }
                 }
                 if (first + kPassScalars * kWave >= hidden) {
-                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
+                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, slot, me), payload_sequence);
                 }
                 uint64_t remaining = destinations;
                 while (remaining) {
@@ -723,8 +737,6 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
                     }
                 }
             }
-            if (hidden == 0 && lane == 0)
-                host_store_release(ack_at(z, state.seg[source], channel, ticket.slot, me), ticket.payload_sequence);
         }
 
         // Row metadata (advanced_layout.cuh:207-215; layout.cuh:31-48).
@@ -752,51 +764,49 @@ __device__ void rx_worker(const DeviceState& state, Queues& q, int channel, int 
             }
         }
         ++reads;
-        if (lane == 0) lds_store(q.rx_retired + worker, ticket_index / state.rx_waves + 1);
+        fence_lds();  // scratch is reused by the next ticket
+        if (lane == 0) device_add(&q.rx_retired[channel].value, 1u);
     }
-    if (lane == 0)
-        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatHostReads),
-                  static_cast<unsigned long long>(reads));
+    if (lane == 0 && reads)
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + kStatHostReads), static_cast<unsigned long long>(reads));
 }
 
+// Workgroup b < C is the control workgroup of channel b (wavefront 0 TX control,
+// wavefront 1 RX control); workgroups b >= C hold payload wavefronts only.  With
+// no payload workgroups configured the control workgroups carry the payload
+// wavefronts themselves.
 template <bool kFp8, bool kVector>
 __global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
-    __shared__ Queues q;
-    int entry_failed = 0;
-    if (threadIdx.x == 0) {
-        entry_failed = load_error_code(state) != 0;
-        q.abort = 0;
-        q.tx_finished = 0;
-        q.rx_finished = 0;
-        q.tx_head = 0;
-        q.rx_head = 0;
-        q.tx_total = -1;
-        q.rx_total = -1;
-        for (int i = 0; i < kMaxTxWaves; ++i) q.tx_done[i] = 0;
-        for (int i = 0; i < kMaxRxWaves; ++i) q.rx_done[i] = q.rx_retired[i] = 0;
+    __shared__ WaveScratch lds;
+    const int channels = state.z.dims.channels;
+    if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) return;
+    const int block = blockIdx.x;
+    int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    uint32_t* scratch = lds.words[wave];
+    TransportQueues& q = *state.queues;
+    if (block < channels) {
+        if (wave == 0) return tx_control(state, q, block, lane);
+        if (wave == 1) return rx_control(state, q, block, lane);
+        if (state.worker_groups > 0) return;
+        wave -= 2;
     }
-    // One immutable entry verdict for the whole workgroup: branching on the
-    // mutable abort flag here could strand a wavefront at the final barrier
-    // (advanced_dispatch.cuh:935-938).
-    if (__syncthreads_or(entry_failed)) return;
-    const int channel = blockIdx.x;
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    if (wave == 0) tx_control(state, q, channel, lane);
-    else if (wave == 1) rx_control(state, q, channel, lane);
-    else if (wave < 2 + state.tx_waves) tx_worker<kFp8, kVector>(state, q, channel, wave - 2, lane);
-    else rx_worker<kFp8, kVector>(state, q, channel, wave - 2 - state.tx_waves, lane);
-    // Every role loop has an explicit completion or abort exit; no workgroup
-    // barrier appears inside a role.
-    __syncthreads();
-    if (threadIdx.x == 0) state.channel_timestamps_ns[channel * 2 + 1] = ticks_to_ns(now_ticks());
+    if (wave < state.tx_waves) tx_worker<kFp8, kVector>(state, q, scratch, lane);
+    else if (wave < state.tx_waves + state.rx_waves) rx_worker<kFp8, kVector>(state, q, scratch, lane);
+    // Every role loop has an explicit completion, abort or timeout exit and no
+    // workgroup barrier follows the entry verdict.
 }
 
 }  // namespace
 
-int transport_threads(int tx_waves, int rx_waves) { return (2 + tx_waves + rx_waves) * kWave; }
+int transport_threads(const DeviceState& state) {
+    const int payload = state.tx_waves + state.rx_waves;
+    const int control = state.worker_groups > 0 ? 2 : 2 + payload;
+    return (control > payload ? control : payload) * kWave;
+}
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
-    const dim3 grid(state.z.dims.channels), block(transport_threads(state.tx_waves, state.rx_waves));
+    const dim3 grid(state.z.dims.channels + state.worker_groups), block(transport_threads(state));
     const bool fp8 = state.z.dims.wire_fp8 != 0;
     // BF16 rows need 16-byte granularity on both sides; FP8 additionally needs
     // whole 16-code vectors on the wire.

@@ -19,14 +19,14 @@ class Config(C.Structure):
     _fields_ = [(name, C.c_int32) for name in (
         "num_ranks", "local_rank", "max_tokens", "hidden", "topk", "num_experts", "channels", "payload_slots",
         "descriptor_slots", "wire_fp8", "timeout_ms", "fuse_receive_expand", "tx_waves", "rx_waves", "peer_threads",
-        "staging_numa_node", "device")] + [("reserved", C.c_int32 * 7)]
+        "staging_numa_node", "device", "worker_groups")] + [("reserved", C.c_int32 * 6)]
 
 
 class Sizes(C.Structure):
     _fields_ = [
         ("unique_rows", C.c_int64), ("expanded_rows", C.c_int64), ("plan_bytes", C.c_int64), ("segment_bytes", C.c_int64),
         ("slot_stride", C.c_int64), ("local_experts", C.c_int32), ("payload_bytes", C.c_int32), ("meta_bytes", C.c_int32),
-        ("mailbox_dwords", C.c_int32), ("transport_threads", C.c_int32), ("reserved", C.c_int32 * 7),
+        ("mailbox_dwords", C.c_int32), ("transport_threads", C.c_int32), ("transport_workgroups", C.c_int32), ("reserved", C.c_int32 * 6),
     ]
 
 

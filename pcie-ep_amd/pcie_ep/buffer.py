@@ -54,6 +54,7 @@ class HostStagedEPBuffer:
         staging_numa_node: int = -1,
         tx_waves: int = 0,
         rx_waves: int = 0,
+        worker_groups: int = 0,
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
@@ -63,6 +64,10 @@ class HostStagedEPBuffer:
         process) is not part of this build.  ``num_ranks`` / ``rank`` give the
         logical world and the rank this GPU plays; ``peer_threads`` the host
         threads standing in for the others (default: one per peer, at most 7).
+        ``worker_groups`` is the number of payload workgroups of the transport
+        kernel and ``tx_waves`` / ``rx_waves`` the payload wavefronts in each (0 =
+        defaults: 48 groups of 1 TX + 2 RX wavefronts; ``worker_groups=-1`` makes
+        the per-channel control workgroups move the rows themselves).
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -115,7 +120,7 @@ class HostStagedEPBuffer:
             peer_threads = min(num_ranks - 1, 7)
         self.runtime = NativeRuntime(rank, num_ranks, num_max_tokens_per_rank, hidden, num_topk, num_experts, self.config,
                                      self.device, peer_threads=peer_threads, staging_numa_node=staging_numa_node,
-                                     tx_waves=tx_waves, rx_waves=rx_waves)
+                                     tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups)
         self.peers = PeerGroup(self.runtime) if peer_threads > 0 and num_ranks > 1 else None
         self._comm_stream.wait_stream(torch.cuda.current_stream(self.device))
 

@@ -67,7 +67,8 @@ class NativeRuntime:
     """Owns one ``pcie_ep_runtime`` plus its preallocated pools."""
 
     def __init__(self, rank: int, world: int, max_tokens: int, hidden: int, topk: int, experts: int, config: HostStagedConfig,
-                 device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0) -> None:
+                 device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0,
+                 worker_groups: int = 0) -> None:
         self._lib = _native.library()
         self.config = config
         self.device = torch.device("cuda", device)
@@ -78,6 +79,7 @@ class NativeRuntime:
             wire_fp8=int(config.wire_dtype == "fp8_e4m3"), timeout_ms=config.timeout_ms,
             fuse_receive_expand=int(config.fuse_receive_expand), tx_waves=tx_waves, rx_waves=rx_waves,
             peer_threads=peer_threads, staging_numa_node=staging_numa_node, device=device,
+            worker_groups=worker_groups,
         )
         self.native_config = native
         self.sizes = _native.Sizes()

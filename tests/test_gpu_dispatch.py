@@ -26,7 +26,7 @@ def make_buffer(world=WORLD, rank=0, tmax=129, hidden=7168, topk=TOPK, experts=E
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config.setdefault("timeout_ms", 5000)
-    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "peer_threads") if key in config}
+    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "peer_threads", "worker_groups") if key in config}
     return HostStagedEPBuffer(num_max_tokens_per_rank=tmax, hidden=hidden, num_topk=topk, num_experts=experts,
                               config=HostStagedConfig(**config), num_ranks=world, rank=rank, **extra)
 
@@ -107,9 +107,10 @@ def test_large_hidden_multi_pass():
 
 
 def test_wave_counts():
-    for tx_waves, rx_waves in ((1, 1), (4, 6)):
-        with make_buffer(hidden=512, channels=4, payload_slots=2, descriptor_slots=2, tx_waves=tx_waves, rx_waves=rx_waves) as buffer:
-            check_case(buffer, f"tx{tx_waves}rx{rx_waves}", [60] * 8)
+    for tx_waves, rx_waves, helpers in ((1, 1, -1), (4, 6, 3), (2, 2, 300)):
+        with make_buffer(hidden=512, channels=4, payload_slots=2, descriptor_slots=2, tx_waves=tx_waves, rx_waves=rx_waves,
+                         worker_groups=helpers) as buffer:
+            check_case(buffer, f"tx{tx_waves}rx{rx_waves}h{helpers}", [60] * 8)
 
 
 def test_invalid_routes_raise_code_two():
