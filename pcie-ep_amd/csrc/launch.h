@@ -8,11 +8,13 @@
 namespace pcie_ep {
 
 // Payload workgroups of the transport kernel (after the C control workgroups)
-// and the TX / RX payload wavefronts each of them carries.  The defaults keep
-// about 1.4 MB of host reads in flight: enough to saturate a Gen5 x16 link,
-// little enough that control-path reads are not queued behind them for long.
+// and the TX / RX payload wavefronts each of them carries.  The defaults put 96
+// RX wavefronts on the chip, each with one 14 KB row in flight: about 1.4 MB of
+// outstanding host reads, enough to keep a Gen5 x16 link busy (measured 95 % of
+// the pinned hipMemcpy rate), little enough that control-path reads are not
+// queued behind them for long.  96 TX wavefronts finish well before RX does.
 constexpr int kDefaultWorkerGroups = 48;
-constexpr int kDefaultTxWaves = 1;
+constexpr int kDefaultTxWaves = 2;
 constexpr int kDefaultRxWaves = 2;
 constexpr int kMaxTxWaves = 4;
 constexpr int kMaxRxWaves = 6;

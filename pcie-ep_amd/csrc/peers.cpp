@@ -326,11 +326,10 @@ void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int chan
         state.slot_token[slot_index] = token;
     }
     Descriptor* descriptor = descriptor_at(z_, own, channel, me_, ordinal);
-    const uint64_t payload_sequence = sequence(epoch, wrong_sequence ? token + 1 : token);
-    descriptor->payload_sequence = payload_sequence;
     descriptor->payload_slot = slot;
-    descriptor->token_index = token;
-    descriptor->rank_ordinal = state.rank_ordinals[size_t(token) * ranks + me_];
+    // The token identifies the payload (its sequence is sequence(epoch, token));
+    // the fault hook publishes a token that does not match the slot's metadata.
+    descriptor->token_index = wrong_sequence ? token + 1 : token;
     release(&descriptor->ready, sequence(epoch, ordinal));
     state.pending_sequence[slot_index] = sequence(epoch, token);
     if (!state.pending_listed[slot_index]) {
@@ -456,7 +455,7 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                 Descriptor* descriptor = descriptor_at(z_, gpu, channel, rank, ordinal);
                 if (acquire(&descriptor->ready) != sequence(epoch, ordinal)) break;
                 const int slot = descriptor->payload_slot, token = descriptor->token_index;
-                const uint64_t payload_sequence = descriptor->payload_sequence;
+                const uint64_t payload_sequence = sequence(epoch, token);
                 if (slot < 0 || slot >= z_.dims.payload_slots || token < 0 || token >= z_.dims.max_tokens) {
                     error = "GPU published a descriptor with an out-of-range slot or token";
                     return false;
@@ -464,7 +463,7 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                 const char* base = slot_at(z_, gpu, channel, slot);
                 SlotMetaHeader header;
                 std::memcpy(&header, base + z_.meta_offset, sizeof header);
-                if (payload_sequence != sequence(epoch, header.token_index) || header.token_index != token) {
+                if (header.token_index != token) {
                     error = "GPU payload sequence does not match its slot metadata (rank " + std::to_string(rank) + ", channel " +
                             std::to_string(channel) + ", ordinal " + std::to_string(ordinal) + ")";
                     return false;
@@ -477,7 +476,7 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                     const char* meta = base + z_.meta_offset;
                     const int32_t* branch = reinterpret_cast<const int32_t*>(meta + kMetaBranchOffset);
                     state.cap_tokens.push_back(token);
-                    state.cap_rank_ordinals.push_back(descriptor->rank_ordinal);
+                    state.cap_rank_ordinals.push_back(reinterpret_cast<const int32_t*>(meta + kMetaRankOrdinalsOffset)[rank]);
                     state.cap_masks.push_back(header.destination_mask);
                     state.cap_scales.push_back(header.scale);
                     state.cap_payload.insert(state.cap_payload.end(), reinterpret_cast<const uint8_t*>(base),

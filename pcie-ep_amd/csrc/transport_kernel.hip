@@ -340,7 +340,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         backoff();
     }
     if (lane == 0) {
-        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatTxStageBusy),
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRingFull),
                   static_cast<unsigned long long>(stage_busy));
         // Only this wavefront writes the channel's mapped abort word.
         if (aborted(q)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
@@ -383,8 +383,10 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
         Descriptor* descriptor = descriptor_at(z, state.seg[member ? source : me], channel, me, want ? ordinal : 0);
-        bool ready = false;
-        if (want) ready = host_load(&descriptor->ready) == sequence(epoch, ordinal);
+        // One 16-byte load brings READY together with the slot and token it guards.
+        u32x4 published = {0u, 0u, 0u, 0u};
+        if (want) published = host_load_b128(host_resource(descriptor, 16), 0);
+        const bool ready = want && (uint64_t(published[0]) | uint64_t(published[1]) << 32) == sequence(epoch, ordinal);
         const uint64_t ready_lanes = __ballot(ready);
         // Descriptors of one source are consumed in order: accept the leading run.
         const uint64_t group = (ready_lanes >> (source < ranks ? source * lookahead : 0)) & group_mask;
@@ -397,13 +399,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             continue;
         }
         const int ticket_index = reserve_tickets(q.rx_tail, __popcll(accepted), lane) + __popcll(accepted & below);
-        int slot = 0, token = 0;
-        uint64_t payload_sequence = 0;
-        if (accept) {
-            slot = host_field_load(&descriptor->payload_slot);
-            token = host_field_load(&descriptor->token_index);
-            payload_sequence = host_field_load(&descriptor->payload_sequence);
-        }
+        const int slot = int(published[2]), token = int(published[3]);
+        const uint64_t payload_sequence = sequence(epoch, token);
         bool pending = accept;
         while (true) {
             if (pending && ring_entry_free(q.rx_taken, epoch, ticket_index)) {
@@ -444,8 +441,10 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         // Diagnostic: when this channel's receive side finished, relative to the
         // channel's start (column 0), next to the transmit side's drain (column 1).
         state.receive_expand_overlap[channel * 2] = ticks_to_ns(now_ticks() - begin);
-        state.channel_stats[channel * kStatFields + kStatMetaOverlap] = iterations;
-        state.channel_stats[channel * kStatFields + kStatTxCreditMiss] = ring_waits;
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxPolls),
+                  static_cast<unsigned long long>(iterations));
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRingFull),
+                  static_cast<unsigned long long>(ring_waits));
         device_store(&q.rx_finished[channel].value, 1u);
     }
 }
@@ -547,12 +546,10 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         // any lane publishes a descriptor (the counters are wave-wide).
         wait_memory_ops();
         if (targeted) {
-            Descriptor* descriptor = descriptor_at(z, own, channel, lane, my_descriptor);
-            host_field_store(&descriptor->payload_sequence, sequence(epoch, token));
-            host_field_store(&descriptor->payload_slot, int32_t(slot));
-            host_field_store(&descriptor->token_index, int32_t(token));
-            host_field_store(&descriptor->rank_ordinal, int32_t(scratch[kMetaRankOrdinalsOffset / 4 + lane]));
-            host_store_release(&descriptor->ready, sequence(epoch, my_descriptor));
+            // READY, slot and token in one 16-byte store: nothing to order inside the entry.
+            const uint64_t ready = sequence(epoch, my_descriptor);
+            const u32x4 entry = {uint32_t(ready), uint32_t(ready >> 32), uint32_t(slot), uint32_t(token)};
+            host_store_b128(host_resource(descriptor_at(z, own, channel, lane, my_descriptor), 16), 0, entry);
         }
         if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
         ++writes;

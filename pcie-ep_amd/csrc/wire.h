@@ -58,10 +58,12 @@ enum StatField : int {
     kStatHostWrites = 0,     // own tokens published to the host ring
     kStatHostReads = 1,      // remote unique rows read from host rings
     kStatDeliveries = 2,     // sum over published tokens of remote destination ranks
-    kStatMetaOverlap = 3,    // event counters, implementation specific
-    kStatRxNotReady = 4,
-    kStatTxCreditMiss = 5,
-    kStatTxStageBusy = 6,
+    // 3..6 are event counters of this implementation (the reference leaves them
+    // implementation specific); they depend on timing and are not compared.
+    kStatRxPolls = 3,        // descriptor polling passes of the RX control wavefronts
+    kStatRxNotReady = 4,     // ... of which found no new descriptor
+    kStatTxCreditMiss = 5,   // TX waits for a payload slot ACK or descriptor credit
+    kStatRingFull = 6,       // control waits for a free entry of a ticket ring
     kStatDescriptors = 7,    // endpoint descriptors published
 };
 
@@ -70,16 +72,23 @@ struct alignas(128) Signal {
     char pad[120];
 };
 
-// One entry of a (source -> destination, channel) notification queue.
-// Source writes everything except `consumed`; the destination writes `consumed`.
+// One entry of a (source -> destination, channel) notification queue.  The
+// first 16 bytes are written by the source with ONE 16-byte store (the GPU) or
+// as fields followed by a release store of `ready` (a CPU), and read by the
+// destination with ONE 16-byte load (the GPU) or an acquire load of `ready`
+// followed by the fields (a CPU): a naturally aligned 16-byte access inside one
+// cache line is a single PCIe transaction and a single coherent snapshot, so
+// `payload_slot` and `token_index` are valid whenever `ready` matches.  The
+// payload sequence of the reference's descriptor is sequence(epoch,
+// token_index) by construction and is not stored separately; the destination's
+// unique-row ordinal travels in the slot metadata.  The destination alone
+// writes `consumed`.
 struct alignas(128) Descriptor {
-    uint64_t ready;             // seq(epoch, ordinal) once the entry is complete
-    uint64_t payload_sequence;  // seq(epoch, token_index)
+    uint64_t ready;  // sequence(epoch, ordinal) once the entry is complete
     int32_t payload_slot;
     int32_t token_index;
-    int32_t rank_ordinal;       // unique-row ordinal at this destination
-    int32_t reserved;
-    uint64_t consumed;          // seq(epoch, ordinal): credit returned by the destination
+    uint64_t reserved[2];
+    uint64_t consumed;  // sequence(epoch, ordinal): credit returned by the destination
     char pad[88];
 };
 static_assert(sizeof(Signal) == 128 && sizeof(Descriptor) == 128, "wire ABI");
