@@ -94,6 +94,8 @@ struct DeviceState {
 
     int32_t* chan_remote_tokens;  // scratch [C, ceil(Tmax / C)]: ring history for slot reuse
     TransportQueues* queues;
+    uint64_t* layout_flags;       // prologue scratch: one epoch-tagged flag per token chunk
+    int32_t* layout_records;      // prologue scratch: per-chunk bin totals
     int worker_groups;            // payload workgroups after the C control workgroups (spread over the XCDs)
     int tx_waves, rx_waves;       // payload wavefronts per payload workgroup
 
@@ -305,7 +307,7 @@ __device__ inline bool any_abort_wave(const DeviceState& state, int lane) {
         const int flag = index % per_rank;
         const uint64_t* signal = flag == 0 ? signal_at(segment, state.z.abort_offset)
                                            : signal_at(segment, state.z.channel_abort_offset, flag - 1);
-        aborted |= load_acquire_system(signal) != 0;
+        aborted |= host_load(signal) != 0;
     }
     return __any(aborted);
 }

@@ -20,8 +20,12 @@ constexpr int kMaxTxWaves = 4;
 constexpr int kMaxRxWaves = 6;
 constexpr int kMaxWorkerGroups = 1024;
 
-// Epoch begin + layout + count publication (one workgroup).
+// Epoch begin + layout + count publication (one workgroup per chunk of tokens).
+// The layout scratch holds prologue_flag_bytes() of zero-initialised chunk
+// flags followed by the per-chunk records.
 hipError_t launch_prologue(const DeviceState& state, hipStream_t stream);
+size_t prologue_flag_bytes(const SegmentLayout& z);
+size_t prologue_scratch_bytes(const SegmentLayout& z);
 // Channel transport: control / TX / RX-scatter wavefront roles, one workgroup per channel.
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream);
 int transport_threads(const DeviceState& state);

@@ -104,6 +104,7 @@ struct pcie_ep_runtime {
     int32_t* chan_remote_tokens = nullptr;
     int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves, worker_groups = kDefaultWorkerGroups;
     TransportQueues* queues = nullptr;
+    char* layout_scratch = nullptr;
     uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
     int counts_ack_skip_source = -1;
     std::unique_ptr<PeerEmulator> peers;
@@ -168,6 +169,8 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.plan_chan_counts = reinterpret_cast<int32_t*>(plan + rt->plan.chan_counts);
     s.plan_chan_remote = reinterpret_cast<int32_t*>(plan + rt->plan.chan_remote);
     s.chan_remote_tokens = rt->chan_remote_tokens;
+    s.layout_flags = reinterpret_cast<uint64_t*>(rt->layout_scratch);
+    s.layout_records = reinterpret_cast<int32_t*>(rt->layout_scratch + prologue_flag_bytes(rt->z));
     s.unique_payload = static_cast<uint16_t*>(a->unique_payload);
     s.unique_topk_idx = a->unique_topk_idx;
     s.unique_topk_weights = a->unique_topk_weights;
@@ -284,6 +287,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (error == hipSuccess) error = hipMemset(rt->chan_remote_tokens, 0, history);
         if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->queues), sizeof(TransportQueues));
         if (error == hipSuccess) error = hipMemset(rt->queues, 0, sizeof(TransportQueues));
+        if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->layout_scratch), prologue_scratch_bytes(rt->z));
+        if (error == hipSuccess) error = hipMemset(rt->layout_scratch, 0, prologue_scratch_bytes(rt->z));
         if (error == hipSuccess) error = hipDeviceSynchronize();
         if (error != hipSuccess) status = set_error(PCIE_EP_E_HIP, "device workspace allocation failed: %s", hipGetErrorString(error));
     }
@@ -293,6 +298,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (rt->epoch) (void)hipFree(rt->epoch);
         if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
         if (rt->queues) (void)hipFree(rt->queues);
+        if (rt->layout_scratch) (void)hipFree(rt->layout_scratch);
         return status;
     }
     if (config->peer_threads > 0 && dims.num_ranks > 1)
@@ -313,6 +319,7 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     if (rt->epoch) (void)hipFree(rt->epoch);
     if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
     if (rt->queues) (void)hipFree(rt->queues);
+    if (rt->layout_scratch) (void)hipFree(rt->layout_scratch);
     for (hipEvent_t mark : rt->marks)
         if (mark) (void)hipEventDestroy(mark);
     delete rt;
