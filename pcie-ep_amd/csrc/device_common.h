@@ -275,8 +275,10 @@ __device__ __forceinline__ uint64_t load_acquire_device(const uint64_t* address)
 __device__ __forceinline__ void store_release_device(uint64_t* address, uint64_t value) {
     __hip_atomic_store(address, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Relaxed: an acquire here would invalidate caches in every wavefront that
+// merely checks whether the dispatch already failed.
 __device__ __forceinline__ int64_t load_error_code(const DeviceState& state) {
-    return __hip_atomic_load(state.errors, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(state.errors, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // First error wins; context fields follow the reference

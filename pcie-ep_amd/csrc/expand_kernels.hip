@@ -171,7 +171,8 @@ __global__ void __launch_bounds__(256) epilogue_kernel(DeviceState state) {
 
 // Stand-alone expand: unique rows -> expert-major rows (dispatch.cuh:8-65).
 // Algorithmic HBM traffic: unique_count rows read + expanded_count rows written
-// (+ 36 bytes of row metadata per expanded row).
+// (+ 36 bytes of row metadata per expanded row).  The payload loads of a row
+// are issued before the (dependent) metadata loads that name its destinations.
 template <bool kVector>
 __global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
     if (load_error_code(state)) return;
@@ -181,8 +182,12 @@ __global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
     const int global_wave = blockIdx.x * waves_per_block + threadIdx.x / kWave;
     const int total_waves = gridDim.x * waves_per_block;
     const int topk = z.dims.topk, local = z.local_experts, hidden = z.dims.hidden;
+    const int vectors = hidden / 8;
     const int64_t unique = *state.unique_count;
     for (int64_t row = global_wave; row < unique; row += total_waves) {
+        const u32x4* source_row = reinterpret_cast<const u32x4*>(state.unique_payload + size_t(row) * hidden);
+        RowVectors pass;
+        if constexpr (kVector) row_load_vectors<true>(pass, source_row, 0, vectors, lane);
         const int source = int(state.unique_source_meta[row * 3]);
         const int token = int(state.unique_source_meta[row * 3 + 1]);
         int expert = -1;
@@ -199,7 +204,21 @@ __global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
             if (lane == 0) record_error(state, kErrExpandedCapacity);
             return;
         }
-        scatter_row<kVector>(state.unique_payload + size_t(row) * hidden, state.expanded_payload, hidden, my_row, lane);
+        if constexpr (kVector) {
+            const uint64_t destinations = __ballot(my_row >= 0);
+            for (int first = 0; first < vectors; first += kPassItems * kWave) {
+                if (first) row_load_vectors<true>(pass, source_row, first, vectors, lane);
+                uint64_t remaining = destinations;
+                while (remaining) {
+                    const int owner = __builtin_ctzll(remaining);
+                    remaining &= remaining - 1;
+                    const int64_t out_row = __shfl(my_row, owner);
+                    row_store_vectors<true>(pass, reinterpret_cast<u32x4*>(state.expanded_payload + size_t(out_row) * hidden), first, vectors, lane);
+                }
+            }
+        } else {
+            scatter_row<false>(state.unique_payload + size_t(row) * hidden, state.expanded_payload, hidden, my_row, lane);
+        }
         if (my_row >= 0) {
             state.expanded_expert_idx[my_row] = expert;
             state.expanded_weights[my_row] = weight;
