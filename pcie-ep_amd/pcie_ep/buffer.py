@@ -66,7 +66,7 @@ class HostStagedEPBuffer:
         threads standing in for the others (default: one per peer, at most 7).
         ``worker_groups`` is the number of payload workgroups of the transport
         kernel and ``tx_waves`` / ``rx_waves`` the payload wavefronts in each (0 =
-        defaults: 48 groups of 1 TX + 2 RX wavefronts; ``worker_groups=-1`` makes
+        defaults: 48 groups of 2 TX + 2 RX wavefronts; ``worker_groups=-1`` makes
         the per-channel control workgroups move the rows themselves).
         """
         if not torch.cuda.is_available():
