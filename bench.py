@@ -40,29 +40,9 @@ def log(*items) -> None:
 
 
 def build_inputs(tokens: int, topk: int, routing: str, heavy_tail: bool):
-    import numpy as np
-    import torch
+    from helpers import baseline_inputs
 
-    inputs = []
-    hot = None
-    if routing == "hotspot":
-        arrays = np.load(ROOT / "tests" / "golden" / "hotspot_20_80_routes.npz", allow_pickle=False)
-        hot = (arrays["indices"], arrays["weights"])
-    for rank in range(WORLD):
-        generator = torch.Generator().manual_seed(20261024 + rank * 104729 + tokens)
-        x = torch.randn(tokens, HIDDEN, generator=generator)
-        if heavy_tail:
-            channels = torch.randperm(HIDDEN, generator=torch.Generator().manual_seed(7))[: HIDDEN // 100]
-            x[:, channels] *= 50.0
-        x = x.to(torch.bfloat16).contiguous()
-        if hot is not None:
-            idx = torch.from_numpy(hot[0][rank, :tokens].copy())
-            weights = torch.from_numpy(hot[1][rank, :tokens].copy())
-        else:
-            idx = torch.rand(tokens, EXPERTS, generator=generator).topk(topk, dim=1).indices.contiguous()
-            weights = torch.softmax(torch.randn(tokens, topk, generator=generator), dim=1).contiguous()
-        inputs.append((x, idx, weights))
-    return inputs
+    return baseline_inputs(tokens, topk, routing, heavy_tail, WORLD, EXPERTS, HIDDEN)
 
 
 def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000):

@@ -316,19 +316,28 @@ __device__ inline bool any_abort_wave(const DeviceState& state, int lane) {
 
 // Bounded failure detection: the local timeout is checked on every call, the
 // remote flags at most every min(1 ms, timeout / 8) (advanced_common.cuh:380-429).
+// Waits for one named signal (counts_ready, the count mailbox) use the plain
+// timeout and report their own code; generic progress waits (ring progress,
+// ticket hand-off) add a quarter, so that when a named signal is missing the
+// specific code is recorded first rather than whichever wait started earliest.
+__device__ __forceinline__ uint64_t progress_timeout_ticks(const DeviceState& state) {
+    return state.timeout_ticks + state.timeout_ticks / 4;
+}
 struct HealthCheck {
     uint64_t start;
     uint64_t next_scan;
     uint64_t interval;
-    __device__ HealthCheck(const DeviceState& state, uint64_t begin) : start(begin) {
+    uint64_t limit;
+    __device__ HealthCheck(const DeviceState& state, uint64_t begin, bool progress_wait = false) : start(begin) {
         const uint64_t cap = 1000 * kTicksPerUs;
         const uint64_t eighth = state.timeout_ticks / 8;
         interval = eighth < cap ? eighth : cap;
         next_scan = begin + interval;
+        limit = progress_wait ? progress_timeout_ticks(state) : state.timeout_ticks;
     }
     __device__ bool poll(const DeviceState& state, int lane) {
         const uint64_t now = now_ticks();
-        if (now - start > state.timeout_ticks) return true;
+        if (now - start > limit) return true;
         // `now` differs slightly per lane; take lane 0's verdict for the scan.
         const int scan = broadcast_first(now >= next_scan ? 1 : 0);
         if (!scan) return false;

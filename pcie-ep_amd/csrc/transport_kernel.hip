@@ -52,7 +52,7 @@ struct WaveScratch {
 struct Deadline {
     uint64_t start;
     __device__ explicit Deadline(uint64_t begin) : start(begin) {}
-    __device__ bool expired(const DeviceState& state) const { return now_ticks() - start > state.timeout_ticks; }
+    __device__ bool expired(const DeviceState& state) const { return now_ticks() - start > progress_timeout_ticks(state); }
 };
 
 __device__ __forceinline__ bool aborted(TransportQueues& q) { return device_load(&q.abort.value) != 0; }
@@ -232,7 +232,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     char* own = state.seg[me];
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
-    HealthCheck health(state, start);
+    HealthCheck health(state, start, true);
     if (lane == 0) state.channel_timestamps_ns[channel * 2] = ticks_to_ns(start);
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;

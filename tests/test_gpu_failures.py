@@ -1,0 +1,119 @@
+"""Bounded failure detection: every protocol wait of the GPU kernels ends with
+the reference's error code when a peer stops cooperating, the failure is
+terminal for the buffer, and every kernel still exits normally (the conditions
+are forced from the host side: an emulated peer withholds a signal or publishes
+a wrong one, or a host-visible abort word is set; nothing faults or hangs).
+
+Codes follow csrc/kernels/host_staged/common.cuh:26-38 of the reference and the
+scenarios its control-plane tests force (tests/test_control_progress.py,
+tests/test_integration.py:262-330).
+"""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from helpers import make_inputs, run_dispatch, verify_dispatch
+from pcie_ep.peers import FAULT_NO_COUNTS_CONSUMED, FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE
+from test_gpu_dispatch import make_buffer
+
+pytestmark = pytest.mark.gpu
+
+WORLD, EXPERTS, TOPK, HIDDEN, TOKENS = 8, 256, 8, 256, 24
+
+
+def small_buffer(**config):
+    config.setdefault("timeout_ms", 300)
+    return make_buffer(tmax=TOKENS, hidden=HIDDEN, channels=2, **config)
+
+
+def failing_dispatch(buffer, inputs, code):
+    """Dispatch once, expect device error ``code``; the buffer must refuse further work."""
+    for source, (x, idx, weights) in enumerate(inputs):
+        if source != buffer.rank_idx:
+            buffer.peers.set_source(source, x, idx, weights)
+    buffer.peers.start(1)
+    x, idx, weights = (item.cuda() for item in inputs[buffer.rank_idx])
+    result = buffer.dispatch(x, idx, weights, do_expand=True)
+    torch.cuda.synchronize()
+    buffer.peers.cancel()
+    error = result[3].error.cpu().tolist()
+    assert error[0] == code, f"expected device error {code}, got {error}"
+    with pytest.raises(RuntimeError, match="GPU error"):
+        buffer.check_errors()
+    with pytest.raises(RuntimeError, match="failed"):
+        buffer.dispatch(x, idx, weights, do_expand=True)
+    return result
+
+
+@pytest.fixture
+def inputs():
+    return make_inputs(WORLD, [TOKENS] * WORLD, HIDDEN, EXPERTS, TOPK, seed=77)
+
+
+def test_missing_counts_ready_is_code_12(inputs):
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(5, FAULT_NO_COUNTS_READY)
+        print("case: rank 5 never publishes counts_ready", flush=True)
+        failing_dispatch(buffer, inputs, 12)
+
+
+def test_unconsumed_count_mailbox_is_code_11(inputs):
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(2, FAULT_NO_COUNTS_CONSUMED)
+        print("case: rank 2 never acknowledges the count mailbox", flush=True)
+        result, _ = run_dispatch(buffer, inputs)  # the first epoch does not need the acknowledgement
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
+        del result
+        failing_dispatch(buffer, inputs, 11)  # the second must not overwrite counts a peer may still read
+
+
+def test_missing_payload_ack_is_code_15(inputs):
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(6, FAULT_NO_LAST_ACK)
+        print("case: rank 6 never acknowledges its last payload slot", flush=True)
+        failing_dispatch(buffer, inputs, 15)
+
+
+def test_wrong_payload_identity_is_code_18(inputs):
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(3, FAULT_WRONG_SEQUENCE)
+        print("case: rank 3 publishes a descriptor that does not match its slot", flush=True)
+        failing_dispatch(buffer, inputs, 18)
+
+
+@pytest.mark.parametrize("which,index", [(0, 0), (1, 1)])
+def test_host_abort_words_are_terminal_code_19(inputs, which, index):
+    with small_buffer() as buffer:
+        print(f"case: abort word {which}/{index} of rank 4 set by the host", flush=True)
+        buffer.runtime.host_signal_store(4, which, index, 1)
+        assert buffer.runtime.host_signal_load(4, which, index) == 1
+        failing_dispatch(buffer, inputs, 19)
+
+
+def test_forced_control_abort_is_code_15(inputs):
+    with small_buffer(timeout_ms=5000) as buffer:
+        print("case: channel 0 control wavefront aborts after 1 us (test hook)", flush=True)
+        buffer.runtime.set_test_control_abort_after_ns(1000)
+        failing_dispatch(buffer, inputs, 15)
+
+
+def test_a_failed_dispatch_marks_the_channel_abort_word(inputs):
+    """The failing GPU publishes its own abort so that peers stop waiting
+    (the reference does this for every terminal error: advanced_common.cuh:299-348)."""
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(1, FAULT_NO_COUNTS_READY)
+        failing_dispatch(buffer, inputs, 12)
+        words = [buffer.runtime.host_signal_load(0, 1, channel) for channel in range(2)]
+        assert any(words), words
+
+
+def test_delay_hooks_do_not_change_results(inputs):
+    """Test-only delays in the TX / RX / scatter / metadata / prefix paths stretch
+    the pipeline without changing any output (tests/test_f2.py:60-99)."""
+    with small_buffer(timeout_ms=5000, payload_slots=2, descriptor_slots=2) as buffer:
+        buffer.runtime.set_test_delays(20_000, 30_000, 40_000, 10_000)
+        buffer.runtime.set_test_prefix_delay_ns(200_000)
+        result, _ = run_dispatch(buffer, inputs)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
