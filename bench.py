@@ -33,6 +33,7 @@ for entry in (ROOT, ROOT / "pcie-ep_amd", ROOT / "tests"):
 
 WORLD, EXPERTS, HIDDEN = 8, 256, 7168
 HBM_PEAK_GBPS = 8000.0
+COPY_BYTES = 1 << 30  # calibration copy: 1 GiB read + 1 GiB written
 
 
 def log(*items) -> None:
@@ -98,6 +99,19 @@ def cpu_baseline(inputs, payload_bytes, budget_s=20.0, fp8=False):
     }
 
 
+def counted_traffic(tokens, topk, routing, wire):
+    """HBM bytes per launch of the expand kernel as counted by rocprofv3 (FETCH_SIZE
+    + WRITE_SIZE, scaled by the calibration copy), from the committed counter
+    summary of exactly this workload; None when there is none."""
+    summary = ROOT / "profiles" / f"expand_kernel_T{tokens}_top{topk}_{routing}_counters.txt"
+    if wire != "bf16" or not summary.exists():
+        return None
+    for line in summary.read_text().splitlines():
+        if line.startswith("hbm_traffic_bytes_per_launch"):
+            return int(line.split("=")[1].strip())
+    return None
+
+
 def measure_expand(inputs, tokens, topk, channels, repeats=20):
     """Stand-alone expand kernel (unique rows -> expert-major rows) against HBM."""
     import torch
@@ -117,17 +131,22 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
         unique, expanded = int(handle.unique_count.cpu()), int(handle.expanded_count.cpu())
         pool = next(pool for pool in buffer.runtime._pools if not pool.idle())
         plan = handle._layout
+        # HIP events on the launch stream around `batch` back-to-back launches:
+        # the per-launch mean then carries no event or launch-gap overhead and is
+        # comparable with the profiler's kernel durations.
         begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        batch = 10
         for _ in range(3):
             buffer.runtime.expand_unique(pool.tensors, plan, 1, False)
         torch.cuda.synchronize()
         durations = []
-        for _ in range(repeats):
+        for _ in range(max(1, repeats // batch) + 1):
             begin.record()
-            buffer.runtime.expand_unique(pool.tensors, plan, 1, False)
+            for _ in range(batch):
+                buffer.runtime.expand_unique(pool.tensors, plan, 1, False)
             end.record()
             end.synchronize()
-            durations.append(begin.elapsed_time(end))
+            durations.append(begin.elapsed_time(end) / batch)
         mean_ms = sum(durations) / len(durations)
         algorithmic = (unique + expanded) * HIDDEN * 2 + expanded * 36
         del result, handle
@@ -152,6 +171,8 @@ def main() -> int:
     parser.add_argument("--skip-cpu-baseline", action="store_true")
     parser.add_argument("--skip-expand", action="store_true")
     parser.add_argument("--skip-verify", action="store_true")
+    parser.add_argument("--expand-only", action="store_true",
+                        help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the dispatch; --gpus {args.gpus} is not supported "
@@ -172,6 +193,15 @@ def main() -> int:
     h2d, d2h = _native.C.c_double(), _native.C.c_double()
     _native.check(_native.library().pcie_ep_measure_pinned_copy(0, 1 << 30, 5, _native.C.byref(h2d), _native.C.byref(d2h)), invalid=RuntimeError)
     log(f"[bench] pinned hipMemcpy peak: H2D {h2d.value:.2f} GB/s, D2H {d2h.value:.2f} GB/s")
+
+    copy_rate = _native.C.c_double()
+    _native.check(_native.library().pcie_ep_measure_device_copy(0, COPY_BYTES, 5, _native.C.byref(copy_rate)), invalid=RuntimeError)
+    log(f"[bench] plain device copy of {COPY_BYTES} bytes: {copy_rate.value:.0f} GB/s read+write")
+    if args.expand_only:
+        record = measure_expand(inputs, tokens, topk, args.channels, repeats=5)
+        record["hbm_copy_GBps"] = copy_rate.value
+        print(json.dumps({"roofline": record}), flush=True)
+        return 0
 
     buffer = make_buffer(tokens, topk, args.wire, args.channels, fuse=True)
     sizes = buffer.runtime.sizes
@@ -230,8 +260,11 @@ def main() -> int:
     mean = lambda values: sum(values) / len(values)
     transport_ms = mean(kernel_ms["transport"])
     dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"]) + mean(kernel_ms["epilogue"])
-    read_bytes = remote_reads * (payload_bytes + meta_bytes + 32)
-    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 40 + remote_reads * 16
+    # Per remote row read: payload + slot metadata + one 16-byte descriptor poll;
+    # per own token written: payload + slot metadata, one 16-byte descriptor per
+    # destination; per remote row: an 8-byte payload ACK and an 8-byte credit.
+    read_bytes = remote_reads * (payload_bytes + meta_bytes + 16)
+    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 16 + remote_reads * 16
     peak = max(h2d.value, d2h.value)
     step_s = ms_per_step * 1e-3
     value = (own_writes + remote_reads) * payload_bytes / step_s / 1e9
@@ -265,6 +298,8 @@ def main() -> int:
     if not args.skip_expand:
         log("[bench] measuring the stand-alone expand kernel")
         record["roofline"] = measure_expand(inputs, tokens, topk, args.channels)
+        record["roofline"]["hbm_copy_GBps"] = copy_rate.value
+        record["roofline"]["traffic"] = counted_traffic(tokens, topk, args.routing, args.wire)
     else:
         record["roofline"] = None
     if not args.skip_cpu_baseline:

@@ -184,6 +184,12 @@ int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds4);
 /* Pinned-copy bandwidth of this box (GB/s, best of `repeats`), the denominator
  * for "% of x16 peak".  No counterpart in the reference. */
 int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, double* h2d_gbps, double* d2h_gbps);
+/* Read+write rate (GB/s, bytes read plus bytes written, best of `repeats`) of a
+ * plain device-to-device copy of `bytes` (a multiple of 16) done by a kernel
+ * with the row movers' access shape: the practical ceiling the expand kernel is
+ * compared with, and a kernel of known traffic for scaling memory counters.
+ * No counterpart in the reference. */
+int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, double* gbps);
 
 /* ---- Host peer emulator ---------------------------------------------------
  * On one GPU the other logical ranks are host threads that follow the ring

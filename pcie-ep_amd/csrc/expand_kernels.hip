@@ -250,6 +250,23 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const uint8_t* codes, c
         dequantize_row<kVector>(codes + size_t(token) * hidden, scales[token], out + size_t(token) * hidden, hidden, lane);
 }
 
+// Plain device copy with the same access shape as the row movers (a wavefront
+// moves 16 KiB: 16 x 16-byte vectors per lane).  It exists to calibrate
+// measurements: the practical HBM ceiling of a read+write stream, and the
+// scale of the memory traffic counters for a kernel whose traffic is known.
+__global__ void __launch_bounds__(256) hbm_copy_kernel(const u32x4* source, u32x4* destination, int64_t vectors) {
+    const int lane = threadIdx.x % kWave;
+    const int waves_per_block = blockDim.x / kWave;
+    const int64_t total_waves = int64_t(gridDim.x) * waves_per_block;
+    const int64_t chunk = int64_t(kPassItems) * kWave;
+    for (int64_t first = (int64_t(blockIdx.x) * waves_per_block + threadIdx.x / kWave) * chunk; first < vectors; first += total_waves * chunk) {
+        const int count = int(vectors - first < chunk ? vectors - first : chunk);
+        RowVectors row;
+        row_load_vectors<true>(row, source + first, 0, count, lane);
+        row_store_vectors<true>(row, destination + first, 0, count, lane);
+    }
+}
+
 int row_grid(int64_t rows) {
     // Four wavefronts per workgroup, one row per wavefront, capped so that the
     // grid-stride loop still spreads over all 256 CUs several times.
@@ -274,6 +291,14 @@ hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
     const dim3 grid(row_grid(unique_capacity(state.z.dims))), block(256);
     if (state.z.dims.hidden % 8 == 0) hipLaunchKernelGGL(expand_kernel<true>, grid, block, 0, stream, state);
     else hipLaunchKernelGGL(expand_kernel<false>, grid, block, 0, stream, state);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream) {
+    const int64_t vectors = bytes / 16;
+    if (vectors <= 0) return hipSuccess;
+    const dim3 grid(row_grid((vectors + kPassItems * kWave - 1) / (kPassItems * kWave))), block(256);
+    hipLaunchKernelGGL(hbm_copy_kernel, grid, block, 0, stream, static_cast<const u32x4*>(source), static_cast<u32x4*>(destination), vectors);
     return hipGetLastError();
 }
 

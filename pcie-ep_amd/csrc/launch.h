@@ -33,6 +33,8 @@ int transport_threads(const DeviceState& state);
 hipError_t launch_epilogue(const DeviceState& state, hipStream_t stream);
 // Stand-alone expand of unique rows into expert-major rows (+ padding).
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
+// Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.
+hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream);
 // Stand-alone FP8 wire kernels.
 hipError_t launch_quantize(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden, hipStream_t stream);
 hipError_t launch_dequantize(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden, hipStream_t stream);

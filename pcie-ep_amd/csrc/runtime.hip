@@ -496,6 +496,41 @@ int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, 
     return 0;
 }
 
+int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, double* gbps) {
+    if (bytes < 16 || bytes % 16 || repeats < 1 || !gbps) return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
+    HIP_TRY(hipSetDevice(device));
+    void *source = nullptr, *destination = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t begin = nullptr, end = nullptr;
+    hipError_t status = hipMalloc(&source, size_t(bytes));
+    if (status == hipSuccess) status = hipMalloc(&destination, size_t(bytes));
+    if (status == hipSuccess) status = hipMemset(source, 1, size_t(bytes));
+    if (status == hipSuccess) status = hipStreamCreate(&stream);
+    if (status == hipSuccess) status = hipEventCreate(&begin);
+    if (status == hipSuccess) status = hipEventCreate(&end);
+    double best = 0.0;
+    for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+        status = hipEventRecord(begin, stream);
+        if (status == hipSuccess) status = launch_copy(source, destination, bytes, stream);
+        if (status == hipSuccess) status = hipEventRecord(end, stream);
+        if (status == hipSuccess) status = hipEventSynchronize(end);
+        float ms = 0.0f;
+        if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
+        if (status == hipSuccess && i > 0 && ms > 0.0f) {
+            const double rate = 2.0 * double(bytes) / (ms * 1e6);  // bytes read + bytes written
+            if (rate > best) best = rate;
+        }
+    }
+    if (begin) (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    if (stream) (void)hipStreamDestroy(stream);
+    if (source) (void)hipFree(source);
+    if (destination) (void)hipFree(destination);
+    if (status != hipSuccess) return set_error(PCIE_EP_E_HIP, "device copy measurement failed: %s", hipGetErrorString(status));
+    *gbps = best;
+    return 0;
+}
+
 // ---- peer emulator -----------------------------------------------------------------
 
 #define NEED_PEERS(rt)                                                                                        \
