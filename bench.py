@@ -159,6 +159,43 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
         buffer.close()
 
 
+def graph_replay_sweep(topk, channels, sizes=(128, 512, 2048, 8192), replays=20):
+    """Cached layout + hipGraph replay: the plan is built by one eager dispatch,
+    the dispatch is captured with that plan, and `replays` GPU-only replays are
+    timed back to back (mean microseconds per replay, by size)."""
+    import torch
+
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    out = {}
+    for tokens in sizes:
+        inputs = build_inputs(tokens, topk, "uniform", False)
+        config = HostStagedConfig(channels=channels, enable_graph=True, timeout_ms=30000)
+        with HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
+                                num_ranks=WORLD, rank=0) as buffer:
+            set_peers(buffer, inputs)
+            x, idx, weights = (item.cuda() for item in inputs[0])
+            buffer.peers.start(1 + 3 + replays)
+            result = buffer.dispatch(x, idx, weights, do_expand=True)
+            cache = buffer.cache_layout(result[3])
+            del result
+            graph = buffer.capture_dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
+            for _ in range(3):
+                graph.replay(async_with_compute_stream=True)
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            for _ in range(replays):
+                graph.replay(async_with_compute_stream=True)
+            torch.cuda.synchronize()
+            out[str(tokens)] = (time.perf_counter() - started) / replays * 1e6
+            buffer.peers.wait(120_000)
+            error = buffer._last_handle.error.cpu().tolist()
+            if any(error):
+                raise RuntimeError(f"graph replay failed at T={tokens}: {error}")
+        log(f"[bench] graph replay T={tokens}: {out[str(tokens)]:.1f} us")
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
@@ -171,6 +208,8 @@ def main() -> int:
     parser.add_argument("--skip-cpu-baseline", action="store_true")
     parser.add_argument("--skip-expand", action="store_true")
     parser.add_argument("--skip-verify", action="store_true")
+    parser.add_argument("--graph-sweep", action="store_true",
+                        help="also time cached-layout hipGraph replays for T in {128, 512, 2048, 8192}")
     parser.add_argument("--expand-only", action="store_true",
                         help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
     args = parser.parse_args()
@@ -208,31 +247,39 @@ def main() -> int:
     payload_bytes, meta_bytes = int(sizes.payload_bytes), int(sizes.meta_bytes)
     set_peers(buffer, inputs)
     x, idx, weights = (item.cuda() for item in inputs[0])
-    total = args.warmup + args.steps + (0 if args.skip_verify else 1)
+    total = args.warmup + 2 * args.steps + (0 if args.skip_verify else 1)
     buffer.peers.start(total)
     buffer.peers.wait_staged(120_000)
     log("[bench] peers staged; warming up")
-    buffer.runtime.set_kernel_timing(True)
     for _ in range(args.warmup):
         result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
         del result
     torch.cuda.synchronize()
-    kernel_ms = {"prologue": [], "transport": [], "epilogue": []}
-    inside_ns = []
+    # Timed region: exactly `steps` dispatches submitted back to back, as a
+    # steady caller would (nothing is read back, the CPU never waits inside).
     started = time.perf_counter()
     for _ in range(args.steps):
         result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+        del result
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # Per-kernel durations: a second pass with HIP events recorded on the launch
+    # stream around every kernel (reading them waits for that dispatch, so this
+    # pass is not the one that is timed as a whole).
+    buffer.runtime.set_kernel_timing(True)
+    kernel_ms = {"prologue": [], "transport": [], "epilogue": []}
+    inside_ns = []
+    for _ in range(args.steps):
+        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
         stamps = result[3].transport_timestamps_ns
-        # Reading the per-kernel events waits for this dispatch only; the next
-        # one is submitted right after, as a steady caller would.
         times = buffer.runtime.kernel_times_ms()
         for name in kernel_ms:
             kernel_ms[name].append(times[name])
         inside_ns.append(stamps.clone())
         del result, stamps
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
-    ms_per_step = elapsed / args.steps * 1e3
     buffer.runtime.set_kernel_timing(False)
     inside_ns = [item.cpu().tolist() for item in inside_ns]
 
@@ -307,6 +354,8 @@ def main() -> int:
         record["cpu_baseline"] = cpu_baseline(inputs, payload_bytes, fp8=args.wire == "fp8")
     else:
         record["cpu_baseline"] = None
+    if args.graph_sweep:
+        record["graph_replay_us"] = graph_replay_sweep(topk, args.channels)
     print(json.dumps(record), flush=True)
     return 0
 
