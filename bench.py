@@ -99,6 +99,12 @@ def cpu_baseline(inputs, payload_bytes, budget_s=20.0, fp8=False):
     }
 
 
+def percentiles(values):
+    ordered = sorted(values)
+    pick = lambda q: ordered[min(len(ordered) - 1, int(round(q * (len(ordered) - 1))))]
+    return [pick(0.5), pick(0.95)]
+
+
 def counted_traffic(tokens, topk, routing, wire):
     """HBM bytes per launch of the expand kernel as counted by rocprofv3 (FETCH_SIZE
     + WRITE_SIZE, scaled by the calibration copy), from the committed counter
@@ -336,6 +342,7 @@ def main() -> int:
         },
         "dispatch_us": ms_per_step * 1e3, "dispatch_gpu_us": dispatch_gpu_ms * 1e3,
         "kernel_us": {name: mean(values) * 1e3 for name, values in kernel_ms.items()},
+        "dispatch_gpu_us_p50_p95": percentiles([1e3 * sum(step) for step in zip(*kernel_ms.values())]),
         "pcie_pct_of_peak": 100.0 * pcie["frac"],
         "logical_GBps": tokens * topk * HIDDEN * 2 / step_s / 1e9,
         "rows": {"own_published": own_writes, "remote_unique": remote_reads, "local_unique": local_unique, "expanded": expanded},

@@ -50,7 +50,7 @@ typedef struct pcie_ep_config {
     int32_t timeout_ms;         /* device-side protocol timeout */
     int32_t fuse_receive_expand;/* 1: receive waves scatter to expert rows; 0: unique rows + expand kernel */
     int32_t tx_waves;           /* payload TX wavefronts per payload workgroup, 0 = default (2) */
-    int32_t rx_waves;           /* payload RX wavefronts per payload workgroup, 0 = default (2) */
+    int32_t rx_waves;           /* payload RX wavefronts per payload workgroup, 0 = default (2; 4 on the FP8 wire) */
     int32_t peer_threads;       /* host threads standing in for the other ranks; 0 = none */
     int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
     int32_t device;             /* HIP device ordinal */

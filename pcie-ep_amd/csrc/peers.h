@@ -62,9 +62,6 @@ private:
         std::vector<float> weights;
         std::vector<uint32_t> mask;
         std::vector<int32_t> rank_ordinals, expert_indices, expert_ordinals, counts;
-        std::vector<uint8_t> codes;
-        std::vector<float> scales;
-        std::vector<uint8_t> quantized;            // per token: codes/scales valid
         std::vector<std::vector<int>> remote;      // per channel: tokens with a remote destination, ascending
         std::vector<int> channel_counts;           // [C][P]
         std::vector<uint64_t> slot_generation;     // [C*Q]: generation whose bytes sit in the slot

@@ -88,6 +88,7 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
     if (c->worker_groups < -1 || c->worker_groups > kMaxWorkerGroups)
         return set_error(PCIE_EP_E_INVALID, "worker_groups must be -1..%d", kMaxWorkerGroups);
     if (c->peer_threads < 0) return set_error(PCIE_EP_E_INVALID, "peer_threads must be non-negative");
+    if (c->staging_numa_node < -1 || c->staging_numa_node >= 1024) return set_error(PCIE_EP_E_INVALID, "staging_numa_node must be -1..1023");
     dims = Dimensions{c->num_ranks, c->max_tokens, c->hidden, c->topk, c->num_experts, c->channels, c->payload_slots, c->descriptor_slots,
                       c->wire_fp8 ? 1 : 0};
     return 0;
@@ -253,6 +254,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     rt->plan = plan_layout(dims);
     if (config->tx_waves) rt->tx_waves = config->tx_waves;
     if (config->rx_waves) rt->rx_waves = config->rx_waves;
+    // FP8 rows are half as long: twice the wavefronts keep the same bytes in flight.
+    else if (config->wire_fp8) rt->rx_waves = 2 * kDefaultRxWaves;
     if (config->worker_groups) rt->worker_groups = config->worker_groups < 0 ? 0 : config->worker_groups;
 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers

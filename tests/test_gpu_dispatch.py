@@ -26,7 +26,7 @@ def make_buffer(world=WORLD, rank=0, tmax=129, hidden=7168, topk=TOPK, experts=E
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config.setdefault("timeout_ms", 5000)
-    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "peer_threads", "worker_groups") if key in config}
+    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "peer_threads", "worker_groups", "staging_numa_node") if key in config}
     return HostStagedEPBuffer(num_max_tokens_per_rank=tmax, hidden=hidden, num_topk=topk, num_experts=experts,
                               config=HostStagedConfig(**config), num_ranks=world, rank=rank, **extra)
 
@@ -111,6 +111,20 @@ def test_wave_counts():
         with make_buffer(hidden=512, channels=4, payload_slots=2, descriptor_slots=2, tx_waves=tx_waves, rx_waves=rx_waves,
                          worker_groups=helpers) as buffer:
             check_case(buffer, f"tx{tx_waves}rx{rx_waves}h{helpers}", [60] * 8)
+
+
+def test_numa_bound_staging_segments():
+    """The pinned segments can be bound to a NUMA node (the far-node staging of the
+    cached-replay configuration); node 0 exists on every box.  Results do not change."""
+    from pcie_ep import _native
+
+    node = _native.library().pcie_ep_device_numa_node(0)
+    print(f"case: staging on NUMA node 0 (the GPU reports node {node})", flush=True)
+    assert node >= -1
+    with make_buffer(hidden=1024, channels=4, staging_numa_node=0) as buffer:
+        check_case(buffer, "numa0", [65] * 8)
+    with pytest.raises(RuntimeError, match="set_mempolicy"):
+        make_buffer(hidden=64, channels=1, staging_numa_node=900)
 
 
 def test_invalid_routes_raise_code_two():
