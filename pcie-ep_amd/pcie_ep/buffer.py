@@ -1,21 +1,34 @@
 """DeepEP-shaped dispatch buffer over the gfx950 runtime.
 
-Public contract of the reference's ``HostStagedEPBuffer``
-(pcie_ep/buffers/ep.py:19-500; API.md): same constructor and ``dispatch``
-arguments, same five-tuple result, same exceptions and messages for rejected
-calls, same stream ordering and pool-reuse protection.
+Public contract of the reference's ``HostStagedEPBuffer`` (pcie_ep/buffers/ep.py:
+19-500; API.md): the constructor and ``dispatch`` take the same arguments,
+``dispatch`` returns the same five items (or one ``EventOverlap`` when
+deferred), rejected calls raise the same exception types with the same
+messages, results are ordered against the caller's streams the same way and a
+result pool is never overwritten while a consumer stream may still read it.
 
 What differs is the world.  This build runs one process with one GPU: the GPU
 plays logical rank ``rank`` of ``num_ranks`` and the other ranks are host
 threads on the same pinned rings (``buffer.peers``).  Construction therefore
 needs no process group; passing a multi-process group raises.
+
+Structure of this module:
+
+* ``_Ordering`` owns the buffer's communication stream and the set of streams
+  that have consumed results; ``submit`` is the single place where work is put
+  on the communication stream (after the producer of the inputs and after every
+  known consumer) and its completion event is recorded.
+* ``HostStagedEPBuffer._launch`` runs one admitted request — eager
+  (``runtime.dispatch``) or a graph replay — through ``_Ordering.submit`` and
+  wraps the outcome (handle, overlap, outputs).  ``dispatch`` and
+  ``GraphDispatch.replay`` are both thin callers of it.
 """
 
 from __future__ import annotations
 
 import itertools
 import threading
-from typing import Any, Optional
+from typing import Any, Callable, Dict, Optional, Tuple
 
 import torch
 
@@ -23,13 +36,62 @@ from .config import HostStagedConfig
 from .handle import HostStagedEPHandle
 from .overlap import EventOverlap, record_tensors
 from .peers import PeerGroup
+from .request import DispatchRequest, admit
 from .runtime import NativeRuntime
 
-_buffer_ids = itertools.count(1)
+_next_buffer_id = itertools.count(1)
 
 
-def _stream_key(stream: Any) -> tuple:
-    return (stream.device.index, int(stream.cuda_stream))
+class _Ordering:
+    """Stream ordering of one buffer."""
+
+    def __init__(self, device: int) -> None:
+        self.device = device
+        self.stream = torch.cuda.Stream(device=device)
+        self.stream.wait_stream(torch.cuda.current_stream(device))
+        self._consumers: Dict[Tuple[int, int], Any] = {}
+        self._guard = threading.Lock()
+
+    @staticmethod
+    def _key(stream: Any) -> Tuple[int, int]:
+        return (stream.device.index, int(stream.cuda_stream))
+
+    def saw_consumer(self, stream: Any) -> None:
+        """A stream has been ordered after a result; later dispatches reuse the
+        result pools only behind that stream's tail, even when the Python tensors
+        are gone by then (the protection of pcie_ep/buffers/ep.py:197-220)."""
+        key = self._key(stream)
+        if key != self._key(self.stream):
+            with self._guard:
+                self._consumers[key] = stream
+
+    def forget(self) -> None:
+        with self._guard:
+            self._consumers.clear()
+
+    def submit(self, work: Callable[[], Any], previous_event: Any = None) -> Tuple[Any, Any, Any]:
+        """Run ``work`` with the communication stream current, ordered after the
+        inputs' producer and all consumers; returns (its value, the completion
+        event, the caller's stream)."""
+        caller = torch.cuda.current_stream(self.device)
+        with torch.cuda.stream(self.stream):
+            ordered = {self._key(self.stream)}
+            if previous_event is None:
+                self.stream.wait_stream(caller)
+                ordered.add(self._key(caller))
+            elif isinstance(previous_event, EventOverlap):
+                previous_event.current_stream_wait()
+            else:
+                self.stream.wait_event(previous_event)
+            with self._guard:
+                consumers = list(self._consumers.items())
+            for key, stream in consumers:
+                if key not in ordered:
+                    self.stream.wait_stream(stream)
+            value = work()
+            done = torch.cuda.Event()
+            done.record(self.stream)
+        return value, done, caller
 
 
 class HostStagedEPBuffer:
@@ -58,16 +120,17 @@ class HostStagedEPBuffer:
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
-        ``group`` / ``control_group`` exist for signature compatibility: with a
-        process group of more than one member this raises, because the
-        multi-process transport (shared /dev/shm segments registered by every
-        process) is not part of this build.  ``num_ranks`` / ``rank`` give the
-        logical world and the rank this GPU plays; ``peer_threads`` the host
-        threads standing in for the others (default: one per peer, at most 7).
-        ``worker_groups`` is the number of payload workgroups of the transport
-        kernel and ``tx_waves`` / ``rx_waves`` the payload wavefronts in each (0 =
-        defaults: 48 groups of 2 TX + 2 RX wavefronts; ``worker_groups=-1`` makes
-        the per-channel control workgroups move the rows themselves).
+        The arguments up to ``explicitly_destroy`` are the reference's.  ``group``
+        / ``control_group`` are accepted for signature compatibility: a process
+        group with more than one member raises, because the multi-process
+        transport is not part of this build.  The rest is specific to this build:
+        ``num_ranks`` / ``rank`` give the logical world and the rank this GPU
+        plays; ``peer_threads`` the host threads standing in for the others
+        (default: one per peer, at most 7); ``staging_numa_node`` binds the pinned
+        rings to a NUMA node; ``worker_groups`` / ``tx_waves`` / ``rx_waves``
+        shape the transport kernel (0 = defaults: 48 payload workgroups of 2 TX +
+        2 RX wavefronts, 4 RX on the FP8 wire; ``worker_groups=-1`` makes the
+        per-channel control workgroups move the rows themselves).
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -76,88 +139,95 @@ class HostStagedEPBuffer:
         if config is not None and host_staged_config is not None:
             raise ValueError("Supply config or host_staged_config, not both")
         self.config = config or host_staged_config or HostStagedConfig()
-        for name, value in (("num_max_tokens_per_rank", num_max_tokens_per_rank), ("hidden", hidden), ("num_topk", num_topk),
-                            ("num_experts", num_experts)):
-            if not isinstance(value, int) or value < 1:
+        dimensions = {"num_max_tokens_per_rank": num_max_tokens_per_rank, "hidden": hidden, "num_topk": num_topk, "num_experts": num_experts}
+        for name, value in dimensions.items():
+            if not isinstance(value, int) or isinstance(value, bool) or value < 1:
                 raise ValueError(f"{name} must be a positive integer")
-        if group is not None or control_group is not None:
-            import torch.distributed as dist
-
-            probe = group if group is not None else control_group
-            if dist.is_initialized() and dist.get_world_size(probe) > 1:
-                raise NotImplementedError(
-                    "This build runs the dispatch of one GPU with host-emulated peers; a multi-process EP group is not supported"
-                )
-        if require_reuse_nccl_comm:
-            raise RuntimeError("No NCCL/RCCL communicator is available to borrow in the single-process build")
-        if self.config.numa_mode == "relay":
-            raise NotImplementedError("NUMA relay workers are not part of this build; use numa_mode='direct'")
+        self._refuse_unsupported_world(group, control_group, require_reuse_nccl_comm)
         if not isinstance(num_ranks, int) or not 1 <= num_ranks <= 16 or not isinstance(rank, int) or not 0 <= rank < num_ranks:
             raise ValueError("num_ranks must be in [1,16] and rank in [0,num_ranks)")
         if num_experts % num_ranks:
             raise ValueError("Experts must be uniformly divisible among EP ranks")
-        self.group = group
-        self.control_group = control_group
+
+        # Identity and dimensions (names are the reference's attributes).
+        self.group, self.control_group = group, control_group
         self.rank_idx, self.num_ranks = rank, num_ranks
         self.global_ranks = tuple(range(num_ranks))
-        self.num_max_tokens_per_rank = num_max_tokens_per_rank
-        self.hidden, self.num_topk, self.num_experts = hidden, num_topk, num_experts
+        self.num_max_tokens_per_rank, self.hidden = num_max_tokens_per_rank, hidden
+        self.num_topk, self.num_experts = num_topk, num_experts
         self.deterministic, self.explicitly_destroy = deterministic, explicitly_destroy
         self.device = torch.cuda.current_device()
-        self.buffer_id = next(_buffer_ids)
+        self.buffer_id = next(_next_buffer_id)
         self.directory = None
         self.nccl_comm, self.comm_reused, self.comm_reuse_status = None, False, "not_an_nccl_group"
-        self._comm_stream = torch.cuda.Stream(device=self.device)
-        self._last_event = None
-        self._last_handle: Optional[HostStagedEPHandle] = None
-        self._generation = 0
-        self._failed = self._closed = False
+
+        # State.
         self._lock = threading.RLock()
-        self._consumer_streams: dict = {}
+        self._generation = 0
+        self._state = "live"  # "live" -> "failed" | "closed"
+        self._last_handle: Optional[HostStagedEPHandle] = None
         self._graph_capture = None
+        self._ordering = _Ordering(self.device)
         self.runtime: Optional[NativeRuntime] = None
-        if peer_threads is None:
-            peer_threads = min(num_ranks - 1, 7)
+        threads = min(num_ranks - 1, 7) if peer_threads is None else peer_threads
         self.runtime = NativeRuntime(rank, num_ranks, num_max_tokens_per_rank, hidden, num_topk, num_experts, self.config,
-                                     self.device, peer_threads=peer_threads, staging_numa_node=staging_numa_node,
+                                     self.device, peer_threads=threads, staging_numa_node=staging_numa_node,
                                      tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups)
-        self.peers = PeerGroup(self.runtime) if peer_threads > 0 and num_ranks > 1 else None
-        self._comm_stream.wait_stream(torch.cuda.current_stream(self.device))
+        self.peers = PeerGroup(self.runtime) if threads > 0 and num_ranks > 1 else None
+
+    def _refuse_unsupported_world(self, group: Any, control_group: Any, reuse_comm: bool) -> None:
+        probe = group if group is not None else control_group
+        if probe is not None:
+            import torch.distributed as dist
+
+            if dist.is_initialized() and dist.get_world_size(probe) > 1:
+                raise NotImplementedError(
+                    "This build runs the dispatch of one GPU with host-emulated peers; a multi-process EP group is not supported"
+                )
+        if reuse_comm:
+            raise RuntimeError("No NCCL/RCCL communicator is available to borrow in the single-process build")
+        if self.config.numa_mode == "relay":
+            raise NotImplementedError("NUMA relay workers are not part of this build; use numa_mode='direct'")
 
     # ---- streams ------------------------------------------------------------------------
     def get_comm_stream(self) -> Any:
-        return self._comm_stream
-
-    def _register_consumer_stream(self, stream: Any) -> None:
-        """Remember a stream that reads results, so a later dispatch orders its
-        writes into the reused pool after that stream's tail even when the
-        Python tensors are already gone (pcie_ep/buffers/ep.py:197-220)."""
-        with self._lock:
-            key = _stream_key(stream)
-            if key != _stream_key(self._comm_stream):
-                self._consumer_streams[key] = stream
-
-    def _wait_for_dispatch_inputs(self, compute: Any, previous_event: Any) -> None:
-        if previous_event is None:
-            self._comm_stream.wait_stream(compute)
-        elif hasattr(previous_event, "current_stream_wait"):
-            previous_event.current_stream_wait()
-        else:
-            self._comm_stream.wait_event(previous_event)
-        done = {_stream_key(self._comm_stream)}
-        if previous_event is None:
-            done.add(_stream_key(compute))
-        for key, stream in self._consumer_streams.items():
-            if key not in done:
-                self._comm_stream.wait_stream(stream)
-                done.add(key)
+        return self._ordering.stream
 
     @staticmethod
     def capture() -> EventOverlap:
-        """Record a producer dependency on the current stream."""
-        event = torch.cuda.Event()
-        event.record(torch.cuda.current_stream())
-        return EventOverlap(event)
+        """A dependency on everything enqueued so far on the current stream, to be
+        passed as ``previous_event``."""
+        marker = torch.cuda.Event()
+        marker.record(torch.cuda.current_stream())
+        return EventOverlap(marker)
+
+    # ---- one admitted request -> outputs --------------------------------------------------
+    def _launch(self, request: DispatchRequest, work: Callable[[], Dict[str, Any]], keep: tuple, previous_event: Any,
+                asynchronous: bool, deferred: bool = False) -> Any:
+        """Put ``work`` (which returns the result dict) on the communication stream
+        and wrap the outcome.  ``keep`` is kept alive until the event is released."""
+        def on_comm_stream() -> Dict[str, Any]:
+            record_tensors(request.inputs, self._ordering.stream)
+            result = work()
+            if request.stats_out is not None:
+                request.stats_out.add_(result["expert_counts"])
+                request.stats_out.record_stream(self._ordering.stream)
+            return result
+
+        result, done, caller = self._ordering.submit(on_comm_stream, previous_event)
+        overlap = EventOverlap(done, (self, request.inputs, request.stats_out, request.cached, result) + keep, self._ordering.saw_consumer)
+        handle = HostStagedEPHandle(self, request.routes, result, request.expand, request.alignment, overlap)
+        self._last_handle = handle
+        outputs = (result["recv_x"], result.get("recv_topk_idx"),
+                   result.get("recv_topk_weights") if request.weights is not None else None, handle)
+        if not asynchronous:
+            caller.wait_event(done)
+            record_tensors(result, caller)
+            self._ordering.saw_consumer(caller)
+        if deferred:
+            overlap.register_hook_after_wait(lambda: outputs)
+            return overlap
+        return (*outputs, overlap)
 
     # ---- dispatch -----------------------------------------------------------------------
     def dispatch(
@@ -183,8 +253,8 @@ class HostStagedEPBuffer:
         defer_epilogue: bool = False,
     ) -> Any:
         """Dispatch BF16 tokens; returns ``(recv_x, recv_idx, recv_weights, handle,
-        event)`` or, with ``defer_epilogue``, only the event whose first wait
-        returns the other four (pcie_ep/buffers/ep.py:229-360).
+        event)`` or, with ``defer_epilogue``, only the event, whose first wait
+        returns the other four.
 
         Only tensor metadata is inspected; GPU memory is never read here and the
         CPU never waits for the GPU.  Shapes of the results are capacities; the
@@ -192,72 +262,33 @@ class HostStagedEPBuffer:
         """
         with self._lock:
             self._check_live()
+            # Options of the DeepEP signature that this transport does not have.
             if do_cpu_sync:
                 raise NotImplementedError("The main path supports do_cpu_sync=False only")
-            if handle is not None:
-                if self.config.stage < 6:
-                    raise NotImplementedError("Cached dispatch replay is an S6 optimization")
-                if topk_idx is not None:
-                    raise ValueError("topk_idx must be None when a cached handle is supplied")
-                topk_idx = handle.topk_idx
+            if handle is not None and self.config.stage < 6:
+                raise NotImplementedError("Cached dispatch replay is an S6 optimization")
+            if handle is not None and topk_idx is not None:
+                raise ValueError("topk_idx must be None when a cached handle is supplied")
             if do_handle_copy or num_qps or num_sms or use_tma_aligned_col_major_sf:
                 raise NotImplementedError("Handle copy, QPs, SM overrides and FP8 scale layouts are unsupported")
             if previous_event is not None and not allocate_on_comm_stream:
                 raise ValueError("previous_event requires allocate_on_comm_stream=True")
             if defer_epilogue and not async_with_compute_stream:
                 raise ValueError("defer_epilogue requires async_with_compute_stream=True")
-            if do_zero_padding and not do_expand:
-                raise ValueError("do_zero_padding is valid only with do_expand=True")
-            if expert_alignment is None:
-                alignment = handle.expert_alignment if handle is not None else 1
-            else:
-                alignment = expert_alignment
-            if not isinstance(alignment, int) or alignment < 1:
-                raise ValueError("expert_alignment must be a positive integer")
             if num_experts not in (None, self.num_experts):
                 raise ValueError("num_experts differs from the prepared buffer")
             if num_max_tokens_per_rank not in (None, self.num_max_tokens_per_rank):
                 raise ValueError("num_max_tokens_per_rank differs from the prepared buffer")
-            self._validate_input(x, "x", torch.bfloat16, (None, self.hidden))
-            self._validate_input(topk_idx, "topk_idx", torch.int64, (x.shape[0], self.num_topk))
-            if x.shape[0] > self.num_max_tokens_per_rank:
-                raise ValueError("Input token count exceeds the prepared capacity")
-            if topk_weights is not None:
-                self._validate_input(topk_weights, "topk_weights", torch.float32, topk_idx.shape)
-            stats_out = cumulative_local_expert_recv_stats
-            if stats_out is not None:
-                self._validate_input(stats_out, "cumulative_local_expert_recv_stats", torch.int32,
-                                     (self.num_experts // self.num_ranks,))
-            cached_layout = handle.validate_cached(self, x, alignment, do_expand) if handle is not None else None
+            request = admit(self, "eager", x, topk_idx, topk_weights, handle=handle, expert_alignment=expert_alignment,
+                            do_expand=do_expand, do_zero_padding=do_zero_padding, stats_out=cumulative_local_expert_recv_stats)
             if torch.cuda.is_current_stream_capturing():
                 raise NotImplementedError("Use capture_dispatch for explicit S6 CUDA Graph preparation")
 
-            compute = torch.cuda.current_stream(self.device)
-            with torch.cuda.stream(self._comm_stream):
-                self._wait_for_dispatch_inputs(compute, previous_event)
-                record_tensors((x, topk_idx, topk_weights), self._comm_stream)
-                result = self.runtime.dispatch(x, topk_idx, topk_weights, self.config.stage, alignment, do_expand,
-                                               do_zero_padding, cached_layout, False)
-                if stats_out is not None:
-                    stats_out.add_(result["expert_counts"])
-                    stats_out.record_stream(self._comm_stream)
-                event = torch.cuda.Event()
-                event.record(self._comm_stream)
+            def eager() -> Dict[str, Any]:
+                return self.runtime.dispatch(request.x, request.routes, request.weights, self.config.stage, request.alignment,
+                                             request.expand, request.zero_padding, request.plan, False)
 
-            keep = (self, x, topk_idx, topk_weights, result, stats_out) + ((handle,) if handle is not None else ())
-            overlap = EventOverlap(event, keep, self._register_consumer_stream)
-            out_handle = HostStagedEPHandle(self, topk_idx, result, do_expand, alignment, overlap)
-            self._last_event, self._last_handle = event, out_handle
-            outputs = (result["recv_x"], result.get("recv_topk_idx"),
-                       result.get("recv_topk_weights") if topk_weights is not None else None, out_handle)
-            if not async_with_compute_stream:
-                compute.wait_event(event)
-                record_tensors(result, compute)
-                self._register_consumer_stream(compute)
-            if defer_epilogue:
-                overlap.register_hook_after_wait(lambda: outputs)
-                return overlap
-            return (*outputs, overlap)
+            return self._launch(request, eager, (), previous_event, async_with_compute_stream, defer_epilogue)
 
     def capture_dispatch(self, *args: Any, **kwargs: Any) -> Any:
         """Prepare the buffer's one fixed-address ``GraphDispatch`` (may synchronise)."""
@@ -270,41 +301,32 @@ class HostStagedEPBuffer:
         self._check_live()
         if self.config.stage < 6:
             raise NotImplementedError("Cached layouts require S6")
-        if handle.buffer_id != self.buffer_id or handle.generation != self._generation:
+        if (handle.buffer_id, handle.generation) != (self.buffer_id, self._generation):
             raise ValueError("The handle belongs to another buffer generation")
         return handle.cache_layout()
 
-    # ---- validation and lifetime -----------------------------------------------------------
-    def _validate_input(self, tensor: Any, name: str, dtype: Any, shape: Any) -> None:
-        if not isinstance(tensor, torch.Tensor):
-            raise TypeError(f"{name} must be a torch Tensor")
-        if not tensor.is_cuda or tensor.device.index != self.device:
-            raise ValueError(f"{name} must be on this buffer's CUDA device")
-        if tensor.dtype != dtype or not tensor.is_contiguous():
-            raise ValueError(f"{name} must be contiguous with dtype {dtype}")
-        matches = tensor.ndim == len(shape) and all(want is None or have == want for have, want in zip(tensor.shape, shape))
-        if not matches:
-            raise ValueError(f"{name} has shape {tuple(tensor.shape)}, expected {tuple(shape)}")
-
+    # ---- lifetime -----------------------------------------------------------------------
     def _check_live(self) -> None:
-        if self._closed or self.runtime is None:
+        if self._state == "closed" or self.runtime is None:
             raise RuntimeError("This buffer is closed")
-        if self._failed:
+        if self._state == "failed":
             raise RuntimeError("This buffer has failed; do not dispatch again")
         if torch.cuda.current_device() != self.device:
             raise RuntimeError("The current CUDA device differs from the buffer's device")
 
     def check_errors(self, handle: Optional[HostStagedEPHandle] = None) -> None:
-        """Explicit diagnostic: waits for the dispatch and reads ``error`` back."""
-        selected = handle or self._last_handle
-        if selected is None:
+        """Explicit diagnostic, the only call that waits for the GPU: synchronises
+        on the dispatch and reads its ``error`` field back.  A device error is
+        terminal for the buffer."""
+        subject = handle if handle is not None else self._last_handle
+        if subject is None:
             return
-        if selected.buffer_id != self.buffer_id or selected.generation != self._generation:
+        if (subject.buffer_id, subject.generation) != (self.buffer_id, self._generation):
             raise ValueError("The handle belongs to a different buffer generation")
-        selected._completion_event.synchronize()
-        codes = selected.error.detach().cpu().reshape(-1).tolist()
+        subject._completion_event.synchronize()
+        codes = subject.error.detach().cpu().reshape(-1).tolist()
         if any(codes):
-            self._failed = True
+            self._state = "failed"
             raise RuntimeError(f"PCIe dispatch GPU error on rank {self.rank_idx}: {codes}")
 
     def combine(self, *args: Any, **kwargs: Any) -> Any:
@@ -313,29 +335,25 @@ class HostStagedEPBuffer:
     def close(self) -> None:
         """Drain the GPU, stop the peer threads and free the pinned rings."""
         with self._lock:
-            if self._closed:
+            if self._state == "closed":
                 return
             if self._graph_capture is not None:
                 self._graph_capture.close()
                 self._graph_capture = None
-            if self._last_event is not None:
-                self._last_event.synchronize()
             torch.cuda.synchronize(self.device)
             if self.runtime is not None:
                 self.runtime.close()
-            self.runtime = None
-            self.peers = None
-            self._closed = True
+            self.runtime, self.peers, self._last_handle = None, None, None
+            self._ordering.forget()
+            self._state = "closed"
             self._generation += 1
-            self._last_handle = None
-            self._consumer_streams.clear()
 
     destroy = close
 
     def __enter__(self) -> "HostStagedEPBuffer":
         return self
 
-    def __exit__(self, exc_type: Any, exc_value: Any, traceback: Any) -> None:
+    def __exit__(self, *exc_info: Any) -> None:
         self.close()
 
 

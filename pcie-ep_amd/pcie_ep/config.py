@@ -1,34 +1,79 @@
 """Construction-time options of the host-staged dispatch buffer.
 
-Field names, defaults and rejection rules follow the reference's
-``HostStagedConfig`` (pcie_ep/config.py:42-129) so existing call sites keep
-working; options that select code this build does not have are still accepted
-where they do not change results (they are recorded and ignored), and rejected
-where they would.
+The option names, their defaults, which combinations are rejected, with which
+exception type and message, are the reference's public contract
+(pcie_ep/config.py:42-129; its tests match on the messages), so existing call
+sites and configuration files keep working.  Options that only choose between
+code paths of the reference that this build does not have are accepted,
+recorded and ignored where results do not depend on them
+(``receive_expand_mode``, ``pipeline_stages``, ``source_fusion``,
+``warp_specialization``, ``replica_slots``), and rejected at buffer construction
+where they would (``numa_mode='relay'``).
+
+The rejection rules are kept as a table (``_RULES``), evaluated in order: each
+entry is a predicate over the config that is true when the config is *bad*, the
+exception to raise and its message.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass, fields
-from typing import Optional, Tuple
+from typing import Callable, Optional, Tuple
 
-_POSITIVE = ("payload_slots", "descriptor_slots", "timeout_ms", "replica_slots")
-_DELAYS = ("metadata_delay_ns", "tx_delay_ns", "rx_delay_ns", "scatter_delay_ns")
-_MODES = ("scalar", "vectorized", "pipelined")
+
+def _int(value) -> bool:
+    return isinstance(value, int) and not isinstance(value, bool)
+
+
+def _at_least(name: str, low: int) -> Callable[["HostStagedConfig"], bool]:
+    return lambda c: not _int(getattr(c, name)) or getattr(c, name) < low
+
+
+def _bad_affinity(c: "HostStagedConfig") -> bool:
+    cpus = c.relay_cpu_affinity
+    return not isinstance(cpus, tuple) or any(not _int(cpu) or cpu < 0 for cpu in cpus)
+
+
+_RULES: Tuple[Tuple[Callable[["HostStagedConfig"], bool], type, str], ...] = (
+    (_at_least("payload_slots", 1), ValueError, "payload_slots must be a positive integer"),
+    (_at_least("descriptor_slots", 1), ValueError, "descriptor_slots must be a positive integer"),
+    (_at_least("timeout_ms", 1), ValueError, "timeout_ms must be a positive integer"),
+    (_at_least("replica_slots", 1), ValueError, "replica_slots must be a positive integer"),
+    (lambda c: c.stage not in (6, 7, 8), ValueError, "stages 1-5 are retired; stage must be 6, 7 or 8"),
+    (lambda c: not _int(c.channels) or not 1 <= c.channels <= 32, ValueError, "channels must be an integer in [1, 32]"),
+    (lambda c: c.pipeline_stages not in (2, 3), ValueError, "pipeline_stages must be 2 or 3"),
+    (lambda c: c.receive_expand_mode not in ("scalar", "vectorized", "pipelined"), ValueError,
+     "receive_expand_mode must be 'scalar', 'vectorized' or 'pipelined'"),
+    (lambda c: c.receive_expand_mode != "scalar" and not (c.fuse_receive_expand and c.warp_specialization), ValueError,
+     "Non-scalar receive expansion requires fuse_receive_expand and warp_specialization"),
+    (lambda c: c.wire_dtype not in ("bf16", "fp8_e4m3"), ValueError, "wire_dtype must be 'bf16' or 'fp8_e4m3'"),
+    (lambda c: c.wire_dtype != "bf16" and c.stage < 7, NotImplementedError, "FP8 wire transport requires S7"),
+    (lambda c: c.numa_mode not in ("direct", "relay"), ValueError, "numa_mode must be 'direct' or 'relay'"),
+    (lambda c: c.numa_mode == "relay" and c.stage < 8, NotImplementedError, "NUMA relay is an S8 optimization"),
+    (lambda c: not _int(c.relay_workers_per_numa) or not 1 <= c.relay_workers_per_numa <= c.channels, ValueError,
+     "relay_workers_per_numa must be an integer in [1, channels]"),
+    (_bad_affinity, ValueError, "relay_cpu_affinity must be a tuple of nonnegative CPU indices"),
+    (lambda c: len(set(c.relay_cpu_affinity)) != len(c.relay_cpu_affinity), ValueError,
+     "relay_cpu_affinity must contain distinct CPU indices"),
+    (lambda c: c.stage < 8 and (c.relay_workers_per_numa != 1 or bool(c.relay_cpu_affinity)), NotImplementedError,
+     "Relay worker configuration requires S8"),
+    (lambda c: not _int(c.output_pool_size) or c.output_pool_size < 2, ValueError, "output_pool_size must be at least two"),
+    (_at_least("metadata_delay_ns", 0), ValueError, "metadata_delay_ns must be a nonnegative integer"),
+    (_at_least("tx_delay_ns", 0), ValueError, "tx_delay_ns must be a nonnegative integer"),
+    (_at_least("rx_delay_ns", 0), ValueError, "rx_delay_ns must be a nonnegative integer"),
+    (_at_least("scatter_delay_ns", 0), ValueError, "scatter_delay_ns must be a nonnegative integer"),
+)
 
 
 @dataclass(frozen=True)
 class HostStagedConfig:
-    """Host transport capacity and protocol selection.
+    """Ring capacities and protocol selection of one buffer.
 
-    payload_slots / descriptor_slots are the per-channel ring capacities Q and
-    L; they bound what is in flight, not the tokens of one dispatch.  ``stage``
-    is a capability gate on one runtime: 6 (BF16 wire), 7 (adds the FP8 wire),
-    8 (accepted; the CPU relay it gates in the reference is not part of this
-    build, so ``numa_mode='relay'`` is rejected at buffer construction).
-    ``wire_dtype='fp8_e4m3'`` sends E4M3FN bytes plus one FP32 scale per token;
-    tensors stay BF16 on both sides.  ``receive_expand_mode`` is kept for
-    compatibility: every mode runs the same wavefront-per-row receive path.
+    ``payload_slots`` (Q) and ``descriptor_slots`` (L) are per-channel ring
+    capacities: they bound what is in flight, not the tokens of one dispatch.
+    ``stage`` is a capability gate: 6 = BF16 wire, 7 adds the FP8 wire
+    (``wire_dtype='fp8_e4m3'``: E4M3FN bytes plus one FP32 scale per token on
+    the wire, BF16 tensors on both sides), 8 is accepted for compatibility.
     """
 
     payload_slots: int = 256
@@ -55,49 +100,19 @@ class HostStagedConfig:
     receive_expand_mode: str = "pipelined"
 
     def __post_init__(self) -> None:
-        def is_int(value) -> bool:
-            return isinstance(value, int) and not isinstance(value, bool)
+        for is_bad, exception, message in _RULES:
+            if is_bad(self):
+                raise exception(message)
 
-        for name in _POSITIVE:
-            if not is_int(getattr(self, name)) or getattr(self, name) < 1:
-                raise ValueError(f"{name} must be a positive integer")
-        if self.stage not in (6, 7, 8):
-            raise ValueError("stages 1-5 are retired; stage must be 6, 7 or 8")
-        if not is_int(self.channels) or not 1 <= self.channels <= 32:
-            raise ValueError("channels must be an integer in [1, 32]")
-        if self.pipeline_stages not in (2, 3):
-            raise ValueError("pipeline_stages must be 2 or 3")
-        if self.receive_expand_mode not in _MODES:
-            raise ValueError("receive_expand_mode must be 'scalar', 'vectorized' or 'pipelined'")
-        if self.receive_expand_mode != "scalar" and not (self.fuse_receive_expand and self.warp_specialization):
-            raise ValueError("Non-scalar receive expansion requires fuse_receive_expand and warp_specialization")
-        if self.wire_dtype not in ("bf16", "fp8_e4m3"):
-            raise ValueError("wire_dtype must be 'bf16' or 'fp8_e4m3'")
-        if self.wire_dtype != "bf16" and self.stage < 7:
-            raise NotImplementedError("FP8 wire transport requires S7")
-        if self.numa_mode not in ("direct", "relay"):
-            raise ValueError("numa_mode must be 'direct' or 'relay'")
-        if self.numa_mode == "relay" and self.stage < 8:
-            raise NotImplementedError("NUMA relay is an S8 optimization")
-        if not is_int(self.relay_workers_per_numa) or not 1 <= self.relay_workers_per_numa <= self.channels:
-            raise ValueError("relay_workers_per_numa must be an integer in [1, channels]")
-        affinity = self.relay_cpu_affinity
-        if not isinstance(affinity, tuple) or any(not is_int(cpu) or cpu < 0 for cpu in affinity):
-            raise ValueError("relay_cpu_affinity must be a tuple of nonnegative CPU indices")
-        if len(set(affinity)) != len(affinity):
-            raise ValueError("relay_cpu_affinity must contain distinct CPU indices")
-        if self.stage < 8 and (self.relay_workers_per_numa != 1 or affinity):
-            raise NotImplementedError("Relay worker configuration requires S8")
-        if self.output_pool_size < 2:
-            raise ValueError("output_pool_size must be at least two")
-        for name in _DELAYS:
-            if not is_int(getattr(self, name)) or getattr(self, name) < 0:
-                raise ValueError(f"{name} must be a nonnegative integer")
+    @property
+    def fp8_wire(self) -> bool:
+        return self.wire_dtype == "fp8_e4m3"
 
     def native_options(self) -> dict:
-        """Every option as a plain dict (what the reference hands to its
-        extension and compares across ranks: pcie_ep/config.py:104-129)."""
+        """All options except ``directory`` as plain values, plus ``payload_dtype``
+        ('bf16' / 'fp8'): the dict the reference passes to its extension and
+        compares across ranks (pcie_ep/config.py:104-129)."""
         options = {item.name: getattr(self, item.name) for item in fields(self) if item.name != "directory"}
         options["relay_cpu_affinity"] = list(self.relay_cpu_affinity)
-        options["payload_dtype"] = "fp8" if self.wire_dtype == "fp8_e4m3" else "bf16"
+        options["payload_dtype"] = "fp8" if self.fp8_wire else "bf16"
         return options

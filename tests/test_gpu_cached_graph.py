@@ -63,7 +63,8 @@ def test_cached_layout_does_not_hold_a_result_pool():
         # keeps its last handle for check_errors).
         assert sum(pool.idle() for pool in buffer.runtime._pools) == 1
         for cache in caches:
-            assert not any(isinstance(value, torch.Tensor) and value is not cache._topk_idx for value in vars(cache).values())
+            held = [getattr(cache._identity, slot) for slot in cache._identity.__slots__]
+            assert [item for item in held if isinstance(item, torch.Tensor)] == [cache.topk_idx]
         _arm(buffer, inputs)
         x, idx, weights = (item.cuda() for item in inputs[0])
         with pytest.raises(RuntimeError, match="route plan pool exhausted"):

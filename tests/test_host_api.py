@@ -191,6 +191,10 @@ def test_cached_layout_keeps_routing_identity_only():
     assert cache.topk_idx is routes and cache._layout == "plan" and cache.buffer_id == 7
     for name in ("unique_count", "expert_counts", "completion", "stats", "source_meta"):
         assert not hasattr(cache, name), name
+    # Nothing but the routing identity: no result tensor can hide in it.
+    assert list(vars(cache)) == ["_identity"]
+    held = [getattr(cache._identity, slot) for slot in cache._identity.__slots__]
+    assert [item for item in held if isinstance(item, torch.Tensor)] == [routes]
     x = torch.zeros(4, 16, dtype=torch.bfloat16)
     assert cache.validate_cached(owner, x, 4, True) == "plan"
     assert handle.validate_cached(owner, x, 4, True) == "plan"
@@ -201,9 +205,9 @@ def test_cached_layout_keeps_routing_identity_only():
     (lambda owner, cache, x: setattr(owner, "buffer_id", 8), ValueError, "another buffer generation"),
     (lambda owner, cache, x: setattr(owner, "global_ranks", (0, 1, 2)), ValueError, "another EP group"),
     (lambda owner, cache, x: setattr(owner, "num_experts", 8), ValueError, "dimensions or expert ownership"),
-    (lambda owner, cache, x: cache._topk_idx.add_(1), RuntimeError, "topk_idx changed"),
-    (lambda owner, cache, x: setattr(cache, "_route_signature", ("moved",)), ValueError, "address, shape or strides"),
-    (lambda owner, cache, x: setattr(cache, "_layout", None), RuntimeError, "immutable cached layout"),
+    (lambda owner, cache, x: cache.topk_idx.add_(1), RuntimeError, "topk_idx changed"),
+    (lambda owner, cache, x: setattr(cache._identity, "routes_signature", ("moved",)), ValueError, "address, shape or strides"),
+    (lambda owner, cache, x: setattr(cache._identity, "plan", None), RuntimeError, "immutable cached layout"),
 ])
 def test_cached_layout_rejections(mutate, exception, fragment):
     handle, owner, _ = make_handle()
@@ -247,3 +251,35 @@ def test_handle_check_errors_delegates_to_the_owner():
     handle, _, _ = make_handle(owner=make_owner(check_errors=seen.append))
     handle.check_errors()
     assert seen == [handle]
+
+
+# ---- admission of a dispatch call (metadata only) -----------------------------------------------
+
+def test_admission_rejections_before_any_gpu_work():
+    from pcie_ep.request import admit, require_tensor
+
+    buffer = SimpleNamespace(device=0, hidden=16, num_topk=2, num_experts=4, num_ranks=2, num_max_tokens_per_rank=8)
+    x = torch.zeros(4, 16, dtype=torch.bfloat16)
+    routes = torch.zeros(4, 2, dtype=torch.int64)
+    with pytest.raises(ValueError, match="positive integer"):
+        admit(buffer, "eager", x, routes, None, expert_alignment=0)
+    with pytest.raises(ValueError, match=r"in \[1,256\]"):
+        admit(buffer, "graph", x, routes, None, expert_alignment=257)
+    with pytest.raises(ValueError, match="positive integer"):
+        admit(buffer, "eager", x, routes, None, expert_alignment=True)
+    with pytest.raises(ValueError, match="valid only with do_expand=True"):
+        admit(buffer, "eager", x, routes, None, do_zero_padding=True)
+    with pytest.raises(ValueError, match="requires do_expand=True"):
+        admit(buffer, "graph", x, routes, None, do_zero_padding=True)
+    with pytest.raises(TypeError, match="x must be a torch Tensor"):
+        admit(buffer, "eager", [1, 2], routes, None)
+    with pytest.raises(ValueError, match="must be on this buffer's CUDA device"):
+        admit(buffer, "eager", x, routes, None)  # CPU tensors are refused, never copied
+    handle, owner, _ = make_handle()
+    with pytest.raises(ValueError, match="topk_idx must be None"):
+        admit(owner, "eager", x, routes, None, handle=handle)
+    # Shape / dtype wording of the tensor check, independent of the device.
+    meta = torch.zeros(4, 3, dtype=torch.int64, device="meta")
+    with pytest.raises(TypeError):
+        require_tensor(None, "topk_idx", 0, torch.int64, (4, 2))
+    assert not meta.is_cuda
