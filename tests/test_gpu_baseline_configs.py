@@ -52,6 +52,21 @@ def test_uniform_top8_t4096():
         del result
 
 
+@pytest.mark.parametrize("slots,descriptors", [(16, 8), (64, 64)])
+def test_ring_wrap_at_scale(slots, descriptors):
+    """T=2048/source with rings far smaller than a channel's tokens (64 per
+    channel): every payload slot and descriptor entry is reused several times
+    in one epoch, in both directions, under full-width rows."""
+    print(f"case: ring wrap T=2048 Q={slots} L={descriptors}", flush=True)
+    inputs = baseline_inputs(2048, 8)
+    with make_buffer(2048, 8, payload_slots=slots, descriptor_slots=descriptors) as buffer:
+        for expand in (True, False):
+            result, _ = run_dispatch(buffer, inputs, expand=expand, capture=True)
+            verify_dispatch(result, inputs, 0, WORLD, EXPERTS, 8, expand, 1, False)
+            verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, 8)
+            del result
+
+
 def test_hotspot_top4_t8192_matches_reference_manifest():
     print("case: hotspot top-4 T=8192 bf16", flush=True)
     inputs = baseline_inputs(8192, 4, "hotspot")
