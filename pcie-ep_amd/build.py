@@ -20,6 +20,7 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OUT_DIR = HERE / "pcie_ep" / "lib"
 LIBRARY = OUT_DIR / "libpcie_ep_amd.so"
+CLIENT = OUT_DIR / "abi_client"
 OBJ_DIR = HERE / "build"
 
 HIP_SOURCES = ["prologue_kernel.hip", "transport_kernel.hip", "expand_kernels.hip", "runtime.hip"]
@@ -61,7 +62,18 @@ def build(force: bool = True) -> Path:
     with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
         objects = list(pool.map(_compile, HIP_SOURCES + CXX_SOURCES))
     _run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-pthread", *map(str, objects), "-o", str(LIBRARY)])
+    build_client()
     return LIBRARY
+
+
+def build_client() -> Path:
+    """The torch-free C++ client of the C ABI (tests/abi_client.cpp): plain g++,
+    the public header, the HIP runtime API and the library, nothing else."""
+    rocm = Path(shutil.which("hipcc")).resolve().parents[1]
+    _run(["g++", "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{rocm / 'include'}", f"-I{HERE.parent / 'include'}",
+          str(HERE.parent / "tests" / "abi_client.cpp"), f"-L{OUT_DIR}", "-lpcie_ep_amd", f"-L{rocm / 'lib'}", "-lamdhip64",
+          "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{rocm / 'lib'}", "-o", str(CLIENT)])
+    return CLIENT
 
 
 if __name__ == "__main__":
