@@ -30,14 +30,6 @@ _I32, _I64, _F32, _BF16 = torch.int32, torch.int64, torch.float32, torch.bfloat1
 _owner_ids = itertools.count(1)
 
 
-def _storage_uses(tensor: torch.Tensor) -> int:
-    return torch._C._storage_Use_Count(tensor.untyped_storage()._cdata)
-
-
-def _references(tensor: torch.Tensor) -> tuple:
-    return sys.getrefcount(tensor), _storage_uses(tensor)
-
-
 class RoutePlan:
     """Opaque immutable routing state (the reference's ``_AdvancedLayout``)."""
 
@@ -48,19 +40,32 @@ class RoutePlan:
 
 
 class _Pool:
+    """One preallocated set of result tensors.
+
+    The pool is busy while anything outside it references one of its tensors:
+    a Python reference to the tensor object (``sys.getrefcount``) or another
+    tensor sharing its storage, such as a view (the storage's use count).  The
+    storage objects are looked up once and kept, so the check is two cheap
+    calls per tensor; the constant references held here are part of the idle
+    baseline.
+    """
+
     def __init__(self, shapes: Dict[str, tuple], device: torch.device) -> None:
         self.tensors: Dict[str, torch.Tensor] = {
             name: torch.empty(shape, dtype=dtype, device=device) for name, (dtype, shape) in shapes.items()
         }
-        self._idle = self._snapshot()
+        self._members = list(self.tensors.values())
+        self._storages = [tensor.untyped_storage() for tensor in self._members]
+        # Output pointers never change: the argument block is filled in once.
+        self.arguments = _native.DispatchArgs(**{name: tensor.data_ptr() for name, tensor in self.tensors.items()})
+        self._idle = self.references()
 
-    def _snapshot(self) -> list:
-        return [_references(self.tensors[name]) for name in self.tensors]
+    def references(self) -> list:
+        use_count = torch._C._storage_Use_Count
+        return [sys.getrefcount(tensor) for tensor in self._members] + [use_count(storage._cdata) for storage in self._storages]
 
     def idle(self) -> bool:
-        """True while nothing outside this pool references any of its tensors
-        (Python objects or views of their storage)."""
-        return self._snapshot() == self._idle
+        return self.references() == self._idle
 
 
 class NativeRuntime:
@@ -163,13 +168,13 @@ class NativeRuntime:
             raise RuntimeError("alignment must be in [1,256]")
         pool = self._select_pool(graph_pool)
         plan = self._select_plan(int(x.shape[0]), cached_layout, graph_pool)
-        arguments = _native.DispatchArgs(
-            x=x.data_ptr(), topk_idx=idx.data_ptr(), topk_weights=weights.data_ptr() if weights is not None else None,
-            num_tokens=int(x.shape[0]), alignment=alignment, expand=int(expand), zero_padding=int(zero_padding),
-            reuse_plan=int(cached_layout is not None), plan=plan.storage.data_ptr(),
-            expanded_capacity_rows=int(self.sizes.expanded_rows),
-            **{name: pool.tensors[name].data_ptr() for name in _native.OUTPUT_POINTERS},
-        )
+        arguments = pool.arguments
+        arguments.x, arguments.topk_idx = x.data_ptr(), idx.data_ptr()
+        arguments.topk_weights = weights.data_ptr() if weights is not None else None
+        arguments.num_tokens, arguments.alignment = int(x.shape[0]), alignment
+        arguments.expand, arguments.zero_padding = int(expand), int(zero_padding)
+        arguments.reuse_plan, arguments.plan = int(cached_layout is not None), plan.storage.data_ptr()
+        arguments.expanded_capacity_rows = int(self.sizes.expanded_rows)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _native.check(self._lib.pcie_ep_dispatch(self._handle, C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
         t = pool.tensors
@@ -191,7 +196,7 @@ class NativeRuntime:
 
     # ---- diagnostics and hooks ----------------------------------------------------------
     def pool_debug(self) -> list:
-        return [[_references(tensor) for tensor in pool.tensors.values()] for pool in self._pools]
+        return [pool.references() for pool in self._pools]
 
     def _require(self) -> C.c_void_p:
         if self._handle is None:
