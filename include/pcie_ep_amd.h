@@ -139,7 +139,11 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* runtime);
 
 /* Replaces AdvancedRuntime::dispatch / launch_dispatch (advanced.hpp:126-156,
  * :472-523): enqueues the dispatch kernels on `stream`, never synchronises and
- * never allocates, so it may be called under stream capture. */
+ * never allocates, so it may be called under stream capture.  Dispatches of one
+ * runtime share its epoch, ticket rings and scratch: they must execute one after
+ * the other (same stream, or streams ordered by events), and calls on one
+ * runtime must not be made from two threads at once (the reference serialises
+ * submissions the same way: pcie_ep/buffers/ep.py:101, :283). */
 int pcie_ep_dispatch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
 
 /* Thread-local message of the last failing call (runtime may be NULL). */
