@@ -125,11 +125,12 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
 
     // ---- stable layout ---------------------------------------------------------------
     uint64_t* masks = reinterpret_cast<uint64_t*>(lds);                       // [W][bins]
-    int* prefix = reinterpret_cast<int*>(masks + size_t(bins) * chunk_waves);  // [W][bins]
-    int* base = prefix + size_t(bins) * chunk_waves;                           // [bins]
+    int* base = reinterpret_cast<int*>(masks + size_t(bins) * chunk_waves);    // [bins]
     int* chan_counts = base + bins;                                            // [C][P]
     int* chan_remote = chan_counts + channels * ranks;                         // [C]
     int* first_error = chan_remote + channels;                                 // lowest token * 64 + branch
+    // Exclusive prefixes inside the chunk never exceed its 1024 tokens: 16 bits each.
+    uint16_t* prefix = reinterpret_cast<uint16_t*>(first_error + 2);           // [W][bins]
     if (!state.reuse_plan && chunk < chunks) {
         for (int i = threadIdx.x; i < bins * chunk_waves; i += blockDim.x) masks[i] = 0;
         for (int i = threadIdx.x; i < channels * ranks; i += blockDim.x) chan_counts[i] = 0;
@@ -182,7 +183,7 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
         for (int bin = threadIdx.x; bin < bins; bin += blockDim.x) {
             int running = 0;
             for (int w = 0; w < chunk_waves; ++w) {
-                prefix[size_t(w) * bins + bin] = running;
+                prefix[size_t(w) * bins + bin] = uint16_t(running);
                 running += __popcll(masks[size_t(w) * bins + bin]);
             }
             device_store(mine + record.counts() + bin, running);
@@ -319,12 +320,15 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
 
 size_t prologue_lds_bytes(const SegmentLayout& z, int chunk_waves) {
     const size_t bins = size_t(z.dims.num_ranks) + z.dims.num_experts;
-    return bins * chunk_waves * 12 + bins * 4 + size_t(z.dims.channels) * z.dims.num_ranks * 4 + size_t(z.dims.channels) * 4 + 64;
+    return bins * chunk_waves * 10 + bins * 4 + size_t(z.dims.channels) * z.dims.num_ranks * 4 + size_t(z.dims.channels) * 4 + 64;
 }
 
+// The largest chunk whose tables fit the 64 KiB of LDS every workgroup may use
+// without opting in to more: 16 wavefronts up to 390 bins, 1 wavefront (14 bytes
+// per bin: 57.6 KB) at the maximum of 16 + 4096 bins.
 int prologue_chunk_waves(const SegmentLayout& z) {
     int waves = 16;
-    while (waves > 1 && prologue_lds_bytes(z, waves) > 144 * 1024) waves /= 2;
+    while (waves > 1 && prologue_lds_bytes(z, waves) > 64 * 1024) waves /= 2;
     return waves;
 }
 
@@ -344,11 +348,7 @@ hipError_t launch_prologue(const DeviceState& state, hipStream_t stream) {
     const int waves = prologue_chunk_waves(state.z);
     const size_t bytes = prologue_lds_bytes(state.z, waves);
     const bool narrow = state.z.dims.topk <= 8;
-    const void* kernel = narrow ? reinterpret_cast<const void*>(prologue_kernel<8>) : reinterpret_cast<const void*>(prologue_kernel<kMaxTopk>);
-    if (bytes > 64 * 1024) {
-        hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (status != hipSuccess) return status;
-    }
+    if (bytes > 64 * 1024) return hipErrorInvalidValue;  // cannot happen within the supported dimensions
     // At least 256 threads so the clear / publish loops stay short.
     const int threads = waves * kWave < 256 ? 256 : waves * kWave;
     const int chunks = state.reuse_plan ? 0 : prologue_chunks(state.z, state.num_tokens);

@@ -113,6 +113,24 @@ def test_wave_counts():
             check_case(buffer, f"tx{tx_waves}rx{rx_waves}h{helpers}", [60] * 8)
 
 
+def test_multi_chunk_layout_with_ragged_token_counts():
+    """The layout kernel cuts tokens into chunks of 1024 (one workgroup each) and
+    chains their totals; token counts that are not multiples of the chunk, differ
+    per rank, or leave the last chunk nearly empty must give the same ordinals."""
+    with make_buffer(tmax=3100, hidden=128, channels=7, payload_slots=32, descriptor_slots=16) as buffer:
+        check_case(buffer, "chunks-ragged", [2500, 3100, 1025, 1, 0, 2048, 1023, 3000], capture=True)
+        check_case(buffer, "chunks-1025", [1025] * 8, expand=False, seed=12)
+        check_case(buffer, "chunks-partial", [3071] * 8, "partial", alignment=16, seed=13)
+
+
+def test_many_experts_narrow_chunks():
+    """With 4096 experts the per-chunk LDS tables only fit two wavefronts of
+    tokens, so a few hundred tokens already span several chained chunks."""
+    with make_buffer(world=16, tmax=700, hidden=64, topk=8, experts=4096, channels=3, payload_slots=8, descriptor_slots=8) as buffer:
+        check_case(buffer, "e4096", [700, 129, 128, 127, 1, 0, 300, 650] * 2)
+        check_case(buffer, "e4096-unique", [333] * 16, expand=False, seed=21)
+
+
 def test_numa_bound_staging_segments():
     """The pinned segments can be bound to a NUMA node (the far-node staging of the
     cached-replay configuration); node 0 exists on every box.  Results do not change."""
