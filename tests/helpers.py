@@ -212,6 +212,8 @@ def verify_captured(peers, inputs: Sequence[Inputs], gpu_rank: int, world: int, 
     if fp8_wire and x.shape[0]:
         codes, scales = fp8_oracle.quantize(x)
         wire, wire_scales = codes.numpy(), scales.numpy()
+    elif fp8_wire:  # no tokens: only the row width matters
+        wire, wire_scales = np.zeros((0, x.shape[1]), np.uint8), np.zeros(0, np.float32)
     else:
         wire, wire_scales = _bits(x).view(np.uint8).reshape(x.shape[0], x.shape[1] * 2), np.ones(x.shape[0], np.float32)
     for rank in range(world):

@@ -1,0 +1,68 @@
+"""Seeded random walk over the configuration space, every case checked bit for
+bit against the oracle: world size and the rank the GPU plays, experts per
+rank, top-k, row length (vector and scalar paths, multi-pass rows), channels,
+ring sizes down to one slot, ragged and empty token counts, both layouts, both
+wires, alignments up to 256, missing weights, route patterns, wavefront counts
+and fused / separate expansion.  Two dispatches per buffer, so slot, descriptor
+and plan reuse across epochs is covered too."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+from helpers import make_inputs, run_dispatch, verify_captured, verify_dispatch
+
+pytestmark = pytest.mark.gpu
+
+
+def draw(case: int) -> dict:
+    rng = random.Random(case)
+    world = rng.choice([1, 2, 3, 4, 5, 8, 8, 8, 12, 16])
+    local = min(rng.choice([1, 2, 3, 4, 8, 32, 32, 64, 256]), 4096 // world)
+    experts = world * local
+    topk = rng.randint(1, min(32, experts))
+    hidden = rng.choice([1, 7, 8, 24, 64, 129, 256, 512, 1000, 2048, 7168, 9000])
+    tmax = rng.choice([1, 5, 33, 64, 65, 200, 1025, 1500])
+    if hidden >= 7168:
+        tmax = min(tmax, 200)
+    expand = rng.random() < 0.7
+    pattern = rng.choice(["random", "random", "random", "partial", "hotspot", "multicast", "local", "none"])
+    if pattern in ("hotspot", "local") and topk > local:
+        pattern = "random"
+    fuse = rng.random() < 0.8
+    return dict(
+        world=world, experts=experts, topk=topk, hidden=hidden, tmax=tmax, expand=expand, pattern=pattern, fuse=fuse,
+        channels=rng.randint(1, 32), slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptors=rng.choice([1, 2, 3, 5, 16, 256]),
+        tokens=[rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)], rank=rng.randrange(world),
+        fp8=rng.random() < 0.3, alignment=rng.choice([1, 1, 2, 8, 16, 128, 256]) if expand else 1, weights=rng.random() < 0.8,
+        waves=rng.choice([(0, 0, 0), (1, 1, -1), (1, 1, 1), (4, 6, 5), (2, 3, 100), (0, 0, 0)]),
+    )
+
+
+@pytest.mark.parametrize("first", range(0, 120, 20))
+def test_random_configurations(first):
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    for case in range(first, first + 20):
+        c = draw(case)
+        print(f"case {case}: {c}", flush=True)
+        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
+                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
+                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
+        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
+                                config=config, num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0], rx_waves=c["waves"][1],
+                                worker_groups=c["waves"][2]) as buffer:
+            for repeat in range(2):
+                inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + repeat,
+                                     gaussian=c["fp8"], heavy_tail=c["fp8"])
+                capture = c["world"] > 1
+                result, _ = run_dispatch(buffer, inputs, expand=c["expand"], alignment=c["alignment"], zero_padding=c["expand"],
+                                         with_weights=c["weights"], capture=capture)
+                verify_dispatch(result, inputs, c["rank"], c["world"], c["experts"], c["topk"], c["expand"], c["alignment"], c["expand"],
+                                with_weights=c["weights"], fp8_wire=c["fp8"])
+                if capture:
+                    verify_captured(buffer.peers, inputs, c["rank"], c["world"], c["experts"], c["topk"], fp8_wire=c["fp8"],
+                                    with_weights=c["weights"])
+                del result
