@@ -34,6 +34,7 @@ for entry in (ROOT, ROOT / "pcie-ep_amd", ROOT / "tests"):
 WORLD, EXPERTS, HIDDEN = 8, 256, 7168
 HBM_PEAK_GBPS = 8000.0
 COPY_BYTES = 1 << 30  # calibration copy: 1 GiB read + 1 GiB written
+HOST_COPY_BYTES = 1 << 29  # kernel-driven pinned copy: 512 MiB each way
 
 
 def log(*items) -> None:
@@ -239,6 +240,11 @@ def main() -> int:
     _native.check(_native.library().pcie_ep_measure_pinned_copy(0, 1 << 30, 5, _native.C.byref(h2d), _native.C.byref(d2h)), invalid=RuntimeError)
     log(f"[bench] pinned hipMemcpy peak: H2D {h2d.value:.2f} GB/s, D2H {d2h.value:.2f} GB/s")
 
+    kernel_read, kernel_write = _native.C.c_double(), _native.C.c_double()
+    _native.check(_native.library().pcie_ep_measure_kernel_host_copy(0, HOST_COPY_BYTES, 3, 96, _native.C.byref(kernel_read),
+                                                                    _native.C.byref(kernel_write)), invalid=RuntimeError)
+    log(f"[bench] kernel-driven pinned copy of {HOST_COPY_BYTES} bytes, 96 wavefronts: read {kernel_read.value:.2f} GB/s, "
+        f"write {kernel_write.value:.2f} GB/s")
     copy_rate = _native.C.c_double()
     _native.check(_native.library().pcie_ep_measure_device_copy(0, COPY_BYTES, 5, _native.C.byref(copy_rate)), invalid=RuntimeError)
     log(f"[bench] plain device copy of {COPY_BYTES} bytes: {copy_rate.value:.0f} GB/s read+write")
@@ -327,6 +333,7 @@ def main() -> int:
         "read_GBps": read_bytes / (transport_ms * 1e-3) / 1e9, "write_GBps": write_bytes / (transport_ms * 1e-3) / 1e9,
         "read_payload_GBps": remote_reads * payload_bytes / (transport_ms * 1e-3) / 1e9,
         "peak_h2d_GBps": h2d.value, "peak_d2h_GBps": d2h.value,
+        "kernel_copy_read_GBps": kernel_read.value, "kernel_copy_write_GBps": kernel_write.value,
         "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d.value,
         "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
     }

@@ -188,6 +188,13 @@ int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds4);
 /* Pinned-copy bandwidth of this box (GB/s, best of `repeats`), the denominator
  * for "% of x16 peak".  No counterpart in the reference. */
 int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, double* h2d_gbps, double* d2h_gbps);
+/* The same between pinned host memory and HBM, but moved by a kernel with
+ * `wavefronts` wavefronts in flight (16 KiB each) through the accesses the
+ * transport kernel uses for host slots: what kernel-initiated traffic can reach
+ * on the host link (host -> device reads, device -> host writes), and a kernel
+ * of known host traffic for scaling counters.  No counterpart in the reference. */
+int pcie_ep_measure_kernel_host_copy(int32_t device, int64_t bytes, int32_t repeats, int32_t wavefronts, double* read_gbps,
+                                     double* write_gbps);
 /* Read+write rate (GB/s, bytes read plus bytes written, best of `repeats`) of a
  * plain device-to-device copy of `bytes` (a multiple of 16) done by a kernel
  * with the row movers' access shape: the practical ceiling the expand kernel is

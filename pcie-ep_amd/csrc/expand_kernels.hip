@@ -267,6 +267,35 @@ __global__ void __launch_bounds__(256) hbm_copy_kernel(const u32x4* source, u32x
     }
 }
 
+// The same copy between pinned host memory and HBM, through the buffer accesses
+// with the system-scope cache policy that the transport kernel uses for host
+// slots.  A fixed number of wavefronts loops over the 16 KiB pieces, so the bytes
+// in flight are wavefronts x 16 KiB as in the transport kernel.  It calibrates
+// what a kernel (as opposed to the copy engine behind hipMemcpy) can pull over
+// the host link, and the scale of the host-traffic counters.
+template <bool kToDevice>
+__global__ void __launch_bounds__(256) host_copy_kernel(char* host, u32x4* device, int64_t vectors) {
+    const int lane = threadIdx.x % kWave;
+    const int waves_per_block = blockDim.x / kWave;
+    const int64_t total_waves = int64_t(gridDim.x) * waves_per_block;
+    const int64_t chunk = int64_t(kPassItems) * kWave;
+    for (int64_t first = (int64_t(blockIdx.x) * waves_per_block + threadIdx.x / kWave) * chunk; first < vectors; first += total_waves * chunk) {
+        const int count = int(vectors - first < chunk ? vectors - first : chunk);
+        const __amdgpu_buffer_rsrc_t piece = host_resource(host + first * 16, uint32_t(count) * 16u);
+        RowVectors row;
+        if constexpr (kToDevice) {
+#pragma unroll
+            for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(piece, uint32_t(j * kWave + lane) * 16u);  // out of range reads 0
+            row_store_vectors<true>(row, device + first, 0, count, lane);
+        } else {
+            row_load_vectors<true>(row, device + first, 0, count, lane);
+#pragma unroll
+            for (int j = 0; j < kPassItems; ++j)
+                if (j * kWave + lane < count) host_store_b128(piece, uint32_t(j * kWave + lane) * 16u, row.v[j]);
+        }
+    }
+}
+
 int row_grid(int64_t rows) {
     // Four wavefronts per workgroup, one row per wavefront, capped so that the
     // grid-stride loop still spreads over all 256 CUs several times.
@@ -299,6 +328,15 @@ hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hip
     if (vectors <= 0) return hipSuccess;
     const dim3 grid(row_grid((vectors + kPassItems * kWave - 1) / (kPassItems * kWave))), block(256);
     hipLaunchKernelGGL(hbm_copy_kernel, grid, block, 0, stream, static_cast<const u32x4*>(source), static_cast<u32x4*>(destination), vectors);
+    return hipGetLastError();
+}
+
+hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_device, int wavefronts, hipStream_t stream) {
+    const int64_t vectors = bytes / 16;
+    if (vectors <= 0) return hipSuccess;
+    const dim3 grid(wavefronts < 4 ? 1 : wavefronts / 4), block(256);
+    if (to_device) hipLaunchKernelGGL(host_copy_kernel<true>, grid, block, 0, stream, static_cast<char*>(host), static_cast<u32x4*>(device), vectors);
+    else hipLaunchKernelGGL(host_copy_kernel<false>, grid, block, 0, stream, static_cast<char*>(host), static_cast<u32x4*>(device), vectors);
     return hipGetLastError();
 }
 

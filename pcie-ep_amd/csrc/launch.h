@@ -35,6 +35,8 @@ hipError_t launch_epilogue(const DeviceState& state, hipStream_t stream);
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
 // Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.
 hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream);
+// Kernel-driven copy between pinned host memory and HBM with `wavefronts` wavefronts in flight.
+hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_device, int wavefronts, hipStream_t stream);
 // Stand-alone FP8 wire kernels.
 hipError_t launch_quantize(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden, hipStream_t stream);
 hipError_t launch_dequantize(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden, hipStream_t stream);

@@ -499,6 +499,45 @@ int pcie_ep_measure_pinned_copy(int32_t device, int64_t bytes, int32_t repeats, 
     return 0;
 }
 
+int pcie_ep_measure_kernel_host_copy(int32_t device, int64_t bytes, int32_t repeats, int32_t wavefronts, double* read_gbps, double* write_gbps) {
+    if (bytes < 16 || bytes % 16 || repeats < 1 || wavefronts < 1 || wavefronts > 65536 || !read_gbps || !write_gbps)
+        return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
+    HIP_TRY(hipSetDevice(device));
+    void *host = nullptr, *dev = nullptr;
+    HIP_TRY(hipHostMalloc(&host, size_t(bytes), hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable));
+    std::memset(host, 1, size_t(bytes));
+    hipStream_t stream = nullptr;
+    hipEvent_t begin = nullptr, end = nullptr;
+    hipError_t status = hipMalloc(&dev, size_t(bytes));
+    if (status == hipSuccess) status = hipStreamCreate(&stream);
+    if (status == hipSuccess) status = hipEventCreate(&begin);
+    if (status == hipSuccess) status = hipEventCreate(&end);
+    double best[2] = {0.0, 0.0};
+    for (int direction = 0; direction < 2 && status == hipSuccess; ++direction) {
+        for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+            status = hipEventRecord(begin, stream);
+            if (status == hipSuccess) status = launch_host_copy(host, dev, bytes, direction == 0, wavefronts, stream);
+            if (status == hipSuccess) status = hipEventRecord(end, stream);
+            if (status == hipSuccess) status = hipEventSynchronize(end);
+            float ms = 0.0f;
+            if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
+            if (status == hipSuccess && i > 0 && ms > 0.0f) {
+                const double rate = double(bytes) / (ms * 1e6);
+                if (rate > best[direction]) best[direction] = rate;
+            }
+        }
+    }
+    if (begin) (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    if (stream) (void)hipStreamDestroy(stream);
+    if (dev) (void)hipFree(dev);
+    (void)hipHostFree(host);
+    if (status != hipSuccess) return set_error(PCIE_EP_E_HIP, "kernel host copy measurement failed: %s", hipGetErrorString(status));
+    *read_gbps = best[0];
+    *write_gbps = best[1];
+    return 0;
+}
+
 int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, double* gbps) {
     if (bytes < 16 || bytes % 16 || repeats < 1 || !gbps) return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
     HIP_TRY(hipSetDevice(device));

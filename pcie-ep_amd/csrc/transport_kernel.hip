@@ -232,7 +232,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     char* own = state.seg[me];
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
-    HealthCheck health(state, start, true);
+    HealthCheck health(state, start, true, channel, channels);
     if (lane == 0) state.channel_timestamps_ns[channel * 2] = ticks_to_ns(start);
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;

@@ -70,6 +70,7 @@ _PROTOTYPES = {
     "pcie_ep_set_kernel_timing": (C.c_int, [C.c_void_p, C.c_int32]),
     "pcie_ep_get_kernel_times": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "pcie_ep_measure_pinned_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "pcie_ep_measure_kernel_host_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "pcie_ep_measure_device_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double)]),
     "pcie_ep_peer_set_source": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
     "pcie_ep_peers_start": (C.c_int, [C.c_void_p, C.c_int32, C.c_uint32]),

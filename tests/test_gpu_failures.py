@@ -109,6 +109,25 @@ def test_a_failed_dispatch_marks_the_channel_abort_word(inputs):
         assert any(words), words
 
 
+def test_guardians_notice_a_peer_abort_long_before_the_timeout(inputs):
+    """While the GPU waits for an acknowledgement that never comes (timeout 20 s),
+    a peer's abort word appears in host memory: the channel guardians, which share
+    the scanning of the abort words, end the dispatch with code 15 within their
+    scan period instead of waiting for the timeout."""
+    import threading
+    import time
+
+    with small_buffer(timeout_ms=20_000) as buffer:
+        buffer.peers.inject_fault(6, FAULT_NO_LAST_ACK)
+        print("case: abort word of rank 3 set by the host 50 ms into a stalled dispatch", flush=True)
+        timer = threading.Timer(0.05, lambda: buffer.runtime.host_signal_store(3, 1, 1, 1))
+        started = time.perf_counter()
+        timer.start()
+        failing_dispatch(buffer, inputs, 15)
+        timer.join()
+        assert time.perf_counter() - started < 5.0
+
+
 def test_delay_hooks_do_not_change_results(inputs):
     """Test-only delays in the TX / RX / scatter / metadata / prefix paths stretch
     the pipeline without changing any output (tests/test_f2.py:60-99)."""
