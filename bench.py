@@ -119,6 +119,20 @@ def counted_traffic(tokens, topk, routing, wire):
     return None
 
 
+def counted_host_traffic(tokens, topk, routing, wire):
+    """Host-link bytes per launch of the transport kernel as counted by the L2's
+    IO request counters (rocprofv3 --pmc, scaled by the kernel-driven pinned
+    copy), from the committed counter summary of exactly this workload."""
+    summary = ROOT / "profiles" / f"transport_kernel_T{tokens}_top{topk}_{routing}_{wire}_counters.txt"
+    found = {"read": None, "write": None}
+    if summary.exists():
+        for line in summary.read_text().splitlines():
+            for direction in found:
+                if line.startswith(f"host_{direction}_traffic_bytes_per_launch"):
+                    found[direction] = int(line.split("=")[1].strip())
+    return found
+
+
 def measure_expand(inputs, tokens, topk, channels, repeats=20):
     """Stand-alone expand kernel (unique rows -> expert-major rows) against HBM."""
     import torch
@@ -337,6 +351,8 @@ def main() -> int:
         "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d.value,
         "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
     }
+    traffic = counted_host_traffic(tokens, topk, args.routing, args.wire)
+    pcie["traffic_read"], pcie["traffic_write"] = traffic["read"], traffic["write"]
     record = {
         "metric": "dispatch PCIe payload GB/s ((U+F_r)*B/t) and us per dispatch, receiver rank 0 of 8",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
