@@ -295,7 +295,7 @@ def main() -> int:
     # stream around every kernel (reading them waits for that dispatch, so this
     # pass is not the one that is timed as a whole).
     buffer.runtime.set_kernel_timing(True)
-    kernel_ms = {"prologue": [], "transport": [], "epilogue": []}
+    kernel_ms = {"prologue": [], "transport": []}
     inside_ns = []
     for _ in range(args.steps):
         result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
@@ -332,7 +332,7 @@ def main() -> int:
 
     mean = lambda values: sum(values) / len(values)
     transport_ms = mean(kernel_ms["transport"])
-    dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"]) + mean(kernel_ms["epilogue"])
+    dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"])
     # Per remote row read: payload + slot metadata + one 16-byte descriptor poll;
     # per own token written: payload + slot metadata, one 16-byte descriptor per
     # destination; per remote row: an 8-byte payload ACK and an 8-byte credit.

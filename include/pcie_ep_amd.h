@@ -179,11 +179,11 @@ int pcie_ep_expand_unique(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args*
 /* Per-kernel timing with HIP events recorded on the dispatch stream (off by
  * default; must stay off for a dispatch that is being captured into a graph).
  * pcie_ep_get_kernel_times waits for the last timed dispatch and returns the
- * milliseconds of {prologue, transport, epilogue, separate expand or 0}.
+ * milliseconds of {prologue, transport, separate expand or 0}.
  * No counterpart in the reference (its harness wraps events around the whole
  * dispatch: benchmarks/benchmark.py:165-198). */
 int pcie_ep_set_kernel_timing(pcie_ep_runtime* runtime, int32_t enable);
-int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds4);
+int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds3);
 
 /* Pinned-copy bandwidth of this box (GB/s, best of `repeats`), the denominator
  * for "% of x16 peak".  No counterpart in the reference. */

@@ -55,6 +55,8 @@ struct alignas(256) TransportQueues {
     QueueCounter rx_tail, tx_tail;  // tickets reserved by producers (fetch-add)
     QueueCounter rx_head, tx_head;  // tickets claimed by workers (fetch-add); .total = tickets of this dispatch
     QueueCounter abort;             // value != 0: every role exits
+    QueueCounter local_head;        // own tokens (then padding gaps) claimed for the local bypass
+    QueueCounter finished;          // role wavefronts that have ended; the last one reduces the statistics
     QueueCounter rx_retired[kMaxChannels], tx_retired[kMaxChannels], rx_finished[kMaxChannels];
     uint64_t rx_ready[kRing], rx_taken[kRing];  // sequence(epoch, n): entry n % kRing holds / has been copied out
     uint64_t tx_ready[kRing], tx_taken[kRing];

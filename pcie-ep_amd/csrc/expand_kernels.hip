@@ -1,13 +1,12 @@
-// HBM-bound kernels of the dispatch: local bypass + padding + statistics
-// (epilogue), the stand-alone expand of unique rows, and the stand-alone FP8
-// wire kernels.  One wavefront moves one row: all 16-byte loads of the row are
-// in flight before the first store, the row is read once and stored to every
-// destination with streaming 16-byte stores.
+// HBM-bound stand-alone kernels: the expand of unique rows into expert-major
+// rows, the FP8 wire kernels and the calibration copies.  One wavefront moves
+// one row: all 16-byte loads of the row are in flight before the first store,
+// the row is read once and stored to every destination with streaming 16-byte
+// stores.
 //
-// Replaces advanced_copy_local_tokens (csrc/kernels/host_staged/advanced_layout.cuh:217-248),
-// advanced_zero_padding (:250-265), advanced_reduce_statistics (:267-283),
-// scatter_expert_inputs (dispatch.cuh:8-65) and quantize_transport_payload
-// (quantization.cuh:34-71).  The reference copies 2 bytes per thread here.
+// Replaces scatter_expert_inputs (csrc/kernels/host_staged/dispatch.cuh:8-65) and
+// quantize_transport_payload (quantization.cuh:34-71).  The reference copies 2
+// bytes per thread here.
 #include "device_common.h"
 #include "launch.h"
 #include "row_codec.h"
@@ -15,159 +14,6 @@
 namespace pcie_ep {
 
 namespace {
-
-// Store one BF16 row (already read into registers pass by pass) to every
-// destination row named by the lanes whose `my_row >= 0`.
-template <bool kVector>
-__device__ inline void scatter_row(const uint16_t* input, uint16_t* output_base, int hidden, int64_t my_row, int lane) {
-    const uint64_t destinations = __ballot(my_row >= 0);
-    if (!destinations) return;
-    if constexpr (kVector) {
-        const int vectors = hidden / 8;
-        const u32x4* source = reinterpret_cast<const u32x4*>(input);
-        for (int first = 0; first < vectors; first += kPassItems * kWave) {
-            RowVectors row;
-            row_load_vectors<true>(row, source, first, vectors, lane);
-            uint64_t remaining = destinations;
-            while (remaining) {
-                const int owner = __builtin_ctzll(remaining);
-                remaining &= remaining - 1;
-                const int64_t out_row = __shfl(my_row, owner);
-                row_store_vectors<true>(row, reinterpret_cast<u32x4*>(output_base + size_t(out_row) * hidden), first, vectors, lane);
-            }
-        }
-    } else {
-        for (int first = 0; first < hidden; first += kPassScalars * kWave) {
-            RowScalars items;
-#pragma unroll
-            for (int j = 0; j < kPassScalars; ++j) {
-                const int index = first + j * kWave + lane;
-                if (index < hidden) items.v[j] = input[index];
-            }
-            uint64_t remaining = destinations;
-            while (remaining) {
-                const int owner = __builtin_ctzll(remaining);
-                remaining &= remaining - 1;
-                uint16_t* output = output_base + size_t(__shfl(my_row, owner)) * hidden;
-#pragma unroll
-                for (int j = 0; j < kPassScalars; ++j) {
-                    const int index = first + j * kWave + lane;
-                    if (index < hidden) output[index] = items.v[j];
-                }
-            }
-        }
-    }
-}
-
-template <bool kVector>
-__device__ inline void zero_row(uint16_t* output, int hidden, int lane) {
-    if constexpr (kVector) {
-        u32x4* destination = reinterpret_cast<u32x4*>(output);
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        for (int index = lane; index < hidden / 8; index += kWave) __builtin_nontemporal_store(zero, destination + index);
-    } else {
-        for (int index = lane; index < hidden; index += kWave) output[index] = 0;
-    }
-}
-
-// Alignment gaps [offset + count, next offset): payload 0, expert -1, weight 0,
-// metadata -1 (advanced_layout.cuh:250-265).
-template <bool kVector>
-__device__ inline void zero_padding_rows(const DeviceState& state, int global_wave, int total_waves, int lane) {
-    const int local = state.z.local_experts, hidden = state.z.dims.hidden;
-    for (int expert = global_wave; expert < local; expert += total_waves) {
-        const int64_t end = state.expert_offsets[expert + 1] < state.expanded_capacity ? state.expert_offsets[expert + 1] : state.expanded_capacity;
-        for (int64_t row = state.expert_prefix[expert]; row < end; ++row) {
-            zero_row<kVector>(state.expanded_payload + size_t(row) * hidden, hidden, lane);
-            if (lane == 0) {
-                state.expanded_expert_idx[row] = -1;
-                state.expanded_weights[row] = 0.0f;
-                state.expanded_source_meta[row * 3] = state.expanded_source_meta[row * 3 + 1] = state.expanded_source_meta[row * 3 + 2] = -1;
-            }
-        }
-    }
-}
-
-template <bool kVector>
-__global__ void __launch_bounds__(256) epilogue_kernel(DeviceState state) {
-    const SegmentLayout& z = state.z;
-    const int lane = threadIdx.x % kWave;
-    const int waves_per_block = blockDim.x / kWave;
-    const int global_wave = blockIdx.x * waves_per_block + threadIdx.x / kWave;
-    const int total_waves = gridDim.x * waves_per_block;
-
-    // Statistics are reduced even after a failure (the reference launches
-    // advanced_reduce_statistics unconditionally).
-    if (global_wave == 0) {
-        const int channels = z.dims.channels;
-        if (lane < kStatFields) {
-            int64_t sum = 0;
-            for (int channel = 0; channel < channels; ++channel) sum += state.channel_stats[channel * kStatFields + lane];
-            state.stats[lane] = sum;
-        }
-        if (lane == 0) {
-            int64_t start = 0, end = 0;
-            for (int channel = 0; channel < channels; ++channel) {
-                const int64_t begin = state.channel_timestamps_ns[channel * 2];
-                if (begin && (!start || begin < start)) start = begin;
-                const int64_t finish = state.channel_timestamps_ns[channel * 2 + 1];
-                if (finish > end) end = finish;
-            }
-            state.transport_timestamps_ns[0] = start;
-            state.transport_timestamps_ns[1] = end;
-        }
-    }
-    if (load_error_code(state)) return;
-
-    // Local bypass: own tokens never touch the host ring and keep the original
-    // BF16 even on an FP8 wire (advanced_layout.cuh:217-248).
-    const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
-    const int hidden = z.dims.hidden;
-    const bool scatter = state.expand && state.fuse_expand;
-    for (int token = global_wave; token < state.num_tokens; token += total_waves) {
-        if (!((state.plan_mask[token] >> me) & 1u)) continue;
-        const uint16_t* input = state.x + size_t(token) * hidden;
-        float weight = 1.0f;
-        int expert_global = -1, ordinal = -1;
-        if (lane < topk) {
-            expert_global = state.plan_exp_idx[size_t(token) * topk + lane];
-            ordinal = state.plan_exp_ord[size_t(token) * topk + lane];
-            if (state.topk_weights) weight = state.topk_weights[size_t(token) * topk + lane];
-        }
-        const int expert = expert_global - me * local;
-        const bool is_local = expert_global >= 0 && expert >= 0 && expert < local;
-        if (scatter) {
-            int64_t my_row = -1;
-            if (is_local) my_row = int64_t(state.expert_offsets[expert]) + state.source_expert_prefix[me * local + expert] + ordinal;
-            if (__any(my_row >= state.expanded_capacity)) {
-                if (lane == 0) record_error(state, kErrExpandedCapacity);
-                return;
-            }
-            scatter_row<kVector>(input, state.expanded_payload, hidden, my_row, lane);
-            if (my_row >= 0) {
-                state.expanded_expert_idx[my_row] = expert;
-                state.expanded_weights[my_row] = weight;
-                state.expanded_source_meta[my_row * 3] = me;
-                state.expanded_source_meta[my_row * 3 + 1] = token;
-                state.expanded_source_meta[my_row * 3 + 2] = lane;
-            }
-        } else {
-            const int64_t row = int64_t(state.source_offsets[me]) + state.plan_rank_ord[size_t(token) * ranks + me];
-            copy_row<kVector, true>(input, state.unique_payload + size_t(row) * hidden, hidden, lane);
-            if (lane < topk) {
-                state.unique_topk_idx[row * topk + lane] = is_local ? expert : -1;
-                state.unique_topk_weights[row * topk + lane] = is_local ? weight : 0.0f;
-                state.unique_expert_ordinals[row * topk + lane] = ordinal;
-            }
-            if (lane == 0) {
-                state.unique_source_meta[row * 3] = me;
-                state.unique_source_meta[row * 3 + 1] = token;
-                state.unique_source_meta[row * 3 + 2] = -1;
-            }
-        }
-    }
-    if (scatter && state.zero_padding) zero_padding_rows<kVector>(state, global_wave, total_waves, lane);
-}
 
 // Stand-alone expand: unique rows -> expert-major rows (dispatch.cuh:8-65).
 // Algorithmic HBM traffic: unique_count rows read + expanded_count rows written
@@ -227,7 +73,8 @@ __global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
             state.expanded_source_meta[my_row * 3 + 2] = lane;
         }
     }
-    if (state.zero_padding) zero_padding_rows<kVector>(state, global_wave, total_waves, lane);
+    if (state.zero_padding)
+        for (int expert = global_wave; expert < local; expert += total_waves) zero_padding_of_expert<kVector>(state, expert, lane);
 }
 
 template <bool kVector>
@@ -306,15 +153,6 @@ int row_grid(int64_t rows) {
 }
 
 }  // namespace
-
-hipError_t launch_epilogue(const DeviceState& state, hipStream_t stream) {
-    int64_t rows = state.num_tokens;
-    if (rows < state.z.local_experts) rows = state.z.local_experts;
-    const dim3 grid(row_grid(rows)), block(256);
-    if (state.z.dims.hidden % 8 == 0) hipLaunchKernelGGL(epilogue_kernel<true>, grid, block, 0, stream, state);
-    else hipLaunchKernelGGL(epilogue_kernel<false>, grid, block, 0, stream, state);
-    return hipGetLastError();
-}
 
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
     const dim3 grid(row_grid(unique_capacity(state.z.dims))), block(256);

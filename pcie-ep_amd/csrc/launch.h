@@ -26,11 +26,10 @@ constexpr int kMaxWorkerGroups = 1024;
 hipError_t launch_prologue(const DeviceState& state, hipStream_t stream);
 size_t prologue_flag_bytes(const SegmentLayout& z);
 size_t prologue_scratch_bytes(const SegmentLayout& z);
-// Channel transport: control / TX / RX-scatter wavefront roles, one workgroup per channel.
+// Channel transport: control / TX / RX-scatter wavefront roles, the local bypass,
+// alignment-gap zeroing and the statistics reduction.
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream);
 int transport_threads(const DeviceState& state);
-// Local bypass copy, alignment-gap zeroing and statistics reduction.
-hipError_t launch_epilogue(const DeviceState& state, hipStream_t stream);
 // Stand-alone expand of unique rows into expert-major rows (+ padding).
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
 // Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.

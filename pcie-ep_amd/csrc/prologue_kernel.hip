@@ -100,8 +100,8 @@ __global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int c
         // Ticket queues of the transport kernel: counters back to zero, totals
         // unknown.  The rings' tags carry the epoch and need no clearing.
         TransportQueues& q = *state.queues;
-        QueueCounter* globals[] = {&q.rx_tail, &q.tx_tail, &q.rx_head, &q.tx_head, &q.abort};
-        if (threadIdx.x < 5) {
+        QueueCounter* globals[] = {&q.rx_tail, &q.tx_tail, &q.rx_head, &q.tx_head, &q.abort, &q.local_head, &q.finished};
+        if (threadIdx.x < 7) {
             globals[threadIdx.x]->value = 0;
             globals[threadIdx.x]->total = -1;
         }

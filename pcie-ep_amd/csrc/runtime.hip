@@ -113,8 +113,8 @@ struct pcie_ep_runtime {
     // Optional per-kernel timing with HIP events on the launch stream.
     bool timing = false;
     bool timing_valid = false;
-    int timing_kernels = 0;
-    hipEvent_t marks[5] = {};
+    bool timing_expand = false;
+    hipEvent_t marks[4] = {};
 };
 
 namespace {
@@ -334,10 +334,11 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     DeviceState state;
     if (int status = build_state(rt, args, state)) return status;
     hipStream_t stream = static_cast<hipStream_t>(stream_handle);
-    // Kernel sequence of launch_dispatch (advanced.hpp:472-523), three launches:
+    // Kernel sequence of launch_dispatch (advanced.hpp:472-523), two launches:
     //   prologue  = begin_epoch + route_flags + stable_ordinals + prepare_channels + publish_counts
-    //   transport = the channel kernel (TX, RX, receive prefixes, fused expand)
-    //   epilogue  = copy_local_tokens + zero_padding + reduce_statistics
+    //   transport = the channel kernel: TX, RX, receive prefixes, fused expand, and - in TX
+    //               wavefronts that have run out of tickets - copy_local_tokens + zero_padding;
+    //               its last wavefront does reduce_statistics
     // and the separate expand when receive/expand fusion is off.
     const bool timed = rt->timing;
     rt->timing_valid = false;
@@ -346,13 +347,11 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     if (timed) HIP_TRY(hipEventRecord(rt->marks[1], stream));
     HIP_TRY(launch_transport(state, stream));
     if (timed) HIP_TRY(hipEventRecord(rt->marks[2], stream));
-    HIP_TRY(launch_epilogue(state, stream));
-    if (timed) HIP_TRY(hipEventRecord(rt->marks[3], stream));
     const bool separate_expand = state.expand && !state.fuse_expand;
     if (separate_expand) HIP_TRY(launch_expand(state, stream));
     if (timed) {
-        HIP_TRY(hipEventRecord(rt->marks[4], stream));
-        rt->timing_kernels = separate_expand ? 4 : 3;
+        HIP_TRY(hipEventRecord(rt->marks[3], stream));
+        rt->timing_expand = separate_expand;
         rt->timing_valid = true;
     }
     return 0;
@@ -370,11 +369,11 @@ int pcie_ep_set_kernel_timing(pcie_ep_runtime* rt, int32_t enable) {
 int pcie_ep_get_kernel_times(pcie_ep_runtime* rt, float* milliseconds) {
     if (!rt || rt->closed || !milliseconds) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
     if (!rt->timing_valid) return set_error(PCIE_EP_E_STATE, "no timed dispatch has been recorded");
-    HIP_TRY(hipEventSynchronize(rt->marks[4]));
-    for (int kernel = 0; kernel < 4; ++kernel) {
-        milliseconds[kernel] = 0.0f;
-        if (kernel < rt->timing_kernels) HIP_TRY(hipEventElapsedTime(milliseconds + kernel, rt->marks[kernel], rt->marks[kernel + 1]));
-    }
+    HIP_TRY(hipEventSynchronize(rt->marks[3]));
+    milliseconds[0] = milliseconds[1] = milliseconds[2] = 0.0f;
+    HIP_TRY(hipEventElapsedTime(milliseconds + 0, rt->marks[0], rt->marks[1]));
+    HIP_TRY(hipEventElapsedTime(milliseconds + 1, rt->marks[1], rt->marks[2]));
+    if (rt->timing_expand) HIP_TRY(hipEventElapsedTime(milliseconds + 2, rt->marks[2], rt->marks[3]));
     return 0;
 }
 

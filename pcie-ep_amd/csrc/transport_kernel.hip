@@ -31,6 +31,13 @@
 //    every control-path read, from the number of channels.
 //  * Workers publish their own descriptors and payload ACKs as soon as their own
 //    stores / loads have completed; control wavefronts only reserve and hand out.
+//  * TX wavefronts run out of tickets long before RX does (the GPU sends one row
+//    per own token and receives P - 1 times as many).  Once the receive prefixes
+//    are known they take over the local bypass (own tokens routed to own experts:
+//    advanced_copy_local_tokens, advanced_layout.cuh:217-248) and the zeroing of
+//    the alignment gaps (:250-265), token by token from a shared counter.  The
+//    last role wavefront to end reduces the per-channel statistics (:267-283).
+//    The dispatch therefore needs no kernel after this one.
 #include "device_common.h"
 #include "launch.h"
 #include "row_codec.h"
@@ -233,7 +240,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
     HealthCheck health(state, start, true, channel, channels);
-    if (lane == 0) state.channel_timestamps_ns[channel * 2] = ticks_to_ns(start);
+    if (lane == 0) device_store(state.channel_timestamps_ns + channel * 2, ticks_to_ns(start));
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;
     const uint64_t below = lanes_below(lane);
@@ -345,7 +352,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         // Only this wavefront writes the channel's mapped abort word.
         if (aborted(q)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
         // Both directions are complete (or aborted): the channel's end time.
-        state.channel_timestamps_ns[channel * 2 + 1] = ticks_to_ns(now_ticks());
+        device_store(state.channel_timestamps_ns + channel * 2 + 1, ticks_to_ns(now_ticks()));
     }
 }
 
@@ -446,6 +453,76 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRingFull),
                   static_cast<unsigned long long>(ring_waits));
         device_store(&q.rx_finished[channel].value, 1u);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Local bypass, padding and the final reduction
+// ---------------------------------------------------------------------------------------
+// Work items: own tokens 0 .. T-1, then (with zero padding on an expanded
+// layout) the local experts' alignment gaps.  Every TX wavefront that has run
+// out of tickets claims items one at a time until none is left.
+template <bool kVector>
+__device__ void local_rows(const DeviceState& state, TransportQueues& q, int lane) {
+    const uint64_t epoch = *state.epoch;
+    // Destination rows depend on the receive prefixes of this epoch.
+    int ready = 0;
+    if (lane == 0) {
+        while (true) {
+            const uint64_t value = load_acquire_device(state.receive_prefix_state + 1);
+            if (value == epoch) { ready = 1; break; }
+            // The wavefront that computes the prefixes owns the timeout.
+            if (value == kPrefixFailed || aborted(q) || load_error_code(state)) break;
+            backoff();
+        }
+    }
+    if (!broadcast_first(ready)) return;
+    const bool padding = state.expand && state.fuse_expand && state.zero_padding;
+    const int items = state.num_tokens + (padding ? state.z.local_experts : 0);
+    while (true) {
+        uint32_t claimed = 0;
+        if (lane == 0) claimed = aborted(q) ? 0xFFFFFFFFu : device_add(&q.local_head.value, 1u);
+        const int item = broadcast_first(int(claimed));
+        if (item < 0 || item >= items) return;
+        if (item >= state.num_tokens) {
+            zero_padding_of_expert<kVector>(state, item - state.num_tokens, lane);
+        } else if (!local_token_rows<kVector>(state, item, lane)) {
+            if (lane == 0) {
+                record_error(state, kErrExpandedCapacity);
+                raise_abort(q);
+            }
+            return;
+        }
+    }
+}
+
+// Called by every role wavefront as its last act.  Everything the reduction
+// reads was written with device-scope stores or atomics, so waiting for this
+// wavefront's own operations is all the ordering the count needs.
+__device__ void finish_role(const DeviceState& state, TransportQueues& q, int lane, uint32_t roles) {
+    wait_memory_ops();
+    uint32_t earlier = 0;
+    if (lane == 0) earlier = device_add(&q.finished.value, 1u);
+    if (uint32_t(broadcast_first(int(earlier))) + 1u != roles) return;
+    // Last one out: column sums of the per-channel statistics and the span of
+    // the channel timestamps.  Done after failures too (the reference launches
+    // advanced_reduce_statistics unconditionally).
+    const int channels = state.z.dims.channels;
+    if (lane < kStatFields) {
+        int64_t sum = 0;
+        for (int channel = 0; channel < channels; ++channel) sum += device_load(state.channel_stats + channel * kStatFields + lane);
+        state.stats[lane] = sum;
+    }
+    if (lane == 0) {
+        int64_t start = 0, end = 0;
+        for (int channel = 0; channel < channels; ++channel) {
+            const int64_t begin = device_load(state.channel_timestamps_ns + channel * 2);
+            if (begin && (!start || begin < start)) start = begin;
+            const int64_t finish = device_load(state.channel_timestamps_ns + channel * 2 + 1);
+            if (finish > end) end = finish;
+        }
+        state.transport_timestamps_ns[0] = start;
+        state.transport_timestamps_ns[1] = end;
     }
 }
 
@@ -566,6 +643,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(deliveries));
         atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(credit_miss));
     }
+    local_rows<kVector>(state, q, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -782,14 +860,21 @@ __global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
     const int lane = threadIdx.x % kWave;
     uint32_t* scratch = lds.words[wave];
     TransportQueues& q = *state.queues;
+    const int payload_waves = state.tx_waves + state.rx_waves;
+    const uint32_t roles = uint32_t(2 * channels + (state.worker_groups > 0 ? state.worker_groups : channels) * payload_waves);
     if (block < channels) {
-        if (wave == 0) return tx_control(state, q, block, lane);
-        if (wave == 1) return rx_control(state, q, block, lane);
+        if (wave < 2) {
+            if (wave == 0) tx_control(state, q, block, lane);
+            else rx_control(state, q, block, lane);
+            return finish_role(state, q, lane, roles);
+        }
         if (state.worker_groups > 0) return;
         wave -= 2;
     }
+    if (wave >= payload_waves) return;
     if (wave < state.tx_waves) tx_worker<kFp8, kVector>(state, q, scratch, lane);
-    else if (wave < state.tx_waves + state.rx_waves) rx_worker<kFp8, kVector>(state, q, scratch, lane);
+    else rx_worker<kFp8, kVector>(state, q, scratch, lane);
+    finish_role(state, q, lane, roles);
     // Every role loop has an explicit completion, abort or timeout exit and no
     // workgroup barrier follows the entry verdict.
 }

@@ -239,9 +239,9 @@ class NativeRuntime:
 
     def kernel_times_ms(self) -> Dict[str, float]:
         """Durations of the last timed dispatch's kernels (waits for it to finish)."""
-        values = (C.c_float * 4)()
+        values = (C.c_float * 3)()
         _native.check(self._lib.pcie_ep_get_kernel_times(self._require(), values), invalid=RuntimeError)
-        return dict(zip(("prologue", "transport", "epilogue", "expand"), (float(v) for v in values)))
+        return dict(zip(("prologue", "transport", "expand"), (float(v) for v in values)))
 
     def pool_tensors(self, index: int) -> Dict[str, torch.Tensor]:
         return self._pools[index].tensors
