@@ -72,7 +72,7 @@ typedef struct pcie_ep_sizes {
     int32_t meta_bytes;         /* per-slot token metadata bytes */
     int32_t mailbox_dwords;
     int32_t transport_threads;  /* workgroup size of the transport kernel */
-    int32_t transport_workgroups;
+    int32_t transport_workgroups; /* control + payload workgroups; 1..32 more do the local bypass */
     int32_t reserved[6];
 } pcie_ep_sizes;
 

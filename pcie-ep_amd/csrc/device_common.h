@@ -100,6 +100,7 @@ struct DeviceState {
     int32_t* layout_records;      // prologue scratch: per-chunk bin totals
     int worker_groups;            // payload workgroups after the C control workgroups (spread over the XCDs)
     int tx_waves, rx_waves;       // payload wavefronts per payload workgroup
+    int local_groups;             // workgroups after those, for the local bypass and padding (>= 1)
 
     uint16_t* unique_payload;
     int64_t* unique_topk_idx;

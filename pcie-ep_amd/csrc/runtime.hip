@@ -149,6 +149,13 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.worker_groups = rt->worker_groups;
     s.tx_waves = rt->tx_waves;
     s.rx_waves = rt->rx_waves;
+    // One local-bypass wavefront per ~8 own tokens, at most 32 workgroups: the work
+    // (HBM only) then ends long before the host link has moved the remote rows.
+    {
+        const int waves_per_group = transport_threads(s) / kWave;
+        const int wanted = (a->num_tokens / 8 + waves_per_group) / waves_per_group;
+        s.local_groups = wanted < 1 ? 1 : (wanted > 32 ? 32 : wanted);
+    }
     s.fuse_expand = rt->config.fuse_receive_expand ? 1 : 0;
     s.expand = a->expand ? 1 : 0;
     s.alignment = a->alignment;

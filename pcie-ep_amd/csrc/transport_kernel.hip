@@ -31,13 +31,13 @@
 //    every control-path read, from the number of channels.
 //  * Workers publish their own descriptors and payload ACKs as soon as their own
 //    stores / loads have completed; control wavefronts only reserve and hand out.
-//  * TX wavefronts run out of tickets long before RX does (the GPU sends one row
-//    per own token and receives P - 1 times as many).  Once the receive prefixes
-//    are known they take over the local bypass (own tokens routed to own experts:
-//    advanced_copy_local_tokens, advanced_layout.cuh:217-248) and the zeroing of
-//    the alignment gaps (:250-265), token by token from a shared counter.  The
-//    last role wavefront to end reduces the per-channel statistics (:267-283).
-//    The dispatch therefore needs no kernel after this one.
+//  * The workgroups after the payload workgroups do the local bypass (own tokens
+//    routed to own experts: advanced_copy_local_tokens, advanced_layout.cuh:217-248)
+//    and the zeroing of the alignment gaps (:250-265) as soon as the receive
+//    prefixes are known, token by token from a shared counter.  That work only
+//    touches HBM and runs on compute units the transport leaves idle, so it hides
+//    completely behind the host link.  The last role wavefront to end reduces the
+//    per-channel statistics (:267-283).  The dispatch needs no kernel after this one.
 #include "device_common.h"
 #include "launch.h"
 #include "row_codec.h"
@@ -460,8 +460,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
 // Local bypass, padding and the final reduction
 // ---------------------------------------------------------------------------------------
 // Work items: own tokens 0 .. T-1, then (with zero padding on an expanded
-// layout) the local experts' alignment gaps.  Every TX wavefront that has run
-// out of tickets claims items one at a time until none is left.
+// layout) the local experts' alignment gaps.  Every wavefront of the local
+// workgroups claims items one at a time until none is left.
 template <bool kVector>
 __device__ void local_rows(const DeviceState& state, TransportQueues& q, int lane) {
     const uint64_t epoch = *state.epoch;
@@ -643,7 +643,6 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(deliveries));
         atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(credit_miss));
     }
-    local_rows<kVector>(state, q, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -861,14 +860,20 @@ __global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
     uint32_t* scratch = lds.words[wave];
     TransportQueues& q = *state.queues;
     const int payload_waves = state.tx_waves + state.rx_waves;
-    const uint32_t roles = uint32_t(2 * channels + (state.worker_groups > 0 ? state.worker_groups : channels) * payload_waves);
+    const int payload_groups = state.worker_groups > 0 ? state.worker_groups : 0;
+    const int waves_per_group = int(blockDim.x) / kWave;
+    const uint32_t roles = uint32_t(2 * channels + (payload_groups ? payload_groups : channels) * payload_waves + state.local_groups * waves_per_group);
+    if (block >= channels + payload_groups) {
+        local_rows<kVector>(state, q, lane);
+        return finish_role(state, q, lane, roles);
+    }
     if (block < channels) {
         if (wave < 2) {
             if (wave == 0) tx_control(state, q, block, lane);
             else rx_control(state, q, block, lane);
             return finish_role(state, q, lane, roles);
         }
-        if (state.worker_groups > 0) return;
+        if (payload_groups) return;
         wave -= 2;
     }
     if (wave >= payload_waves) return;
@@ -888,7 +893,7 @@ int transport_threads(const DeviceState& state) {
 }
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
-    const dim3 grid(state.z.dims.channels + state.worker_groups), block(transport_threads(state));
+    const dim3 grid(state.z.dims.channels + (state.worker_groups > 0 ? state.worker_groups : 0) + state.local_groups), block(transport_threads(state));
     const bool fp8 = state.z.dims.wire_fp8 != 0;
     // BF16 rows need 16-byte granularity on both sides; FP8 additionally needs
     // whole 16-code vectors on the wire.
