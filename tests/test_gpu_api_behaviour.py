@@ -188,3 +188,41 @@ def test_lifetime(inputs):
             other.dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
         with pytest.raises(ValueError, match="another buffer generation"):
             other.cache_layout(handle)
+
+
+def test_dispatch_overlaps_with_compute_on_another_stream():
+    """The dispatch spins on host flags and device counters inside long-running
+    kernels; it must stay correct (and finish) while GEMMs of the caller's stream
+    compete for the compute units, as they do when communication is overlapped
+    with expert computation."""
+    from helpers import baseline_inputs
+
+    tokens = 2048
+    inputs = baseline_inputs(tokens, 8)
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    with HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=7168, num_topk=8, num_experts=256,
+                            config=HostStagedConfig(channels=32, timeout_ms=20_000), num_ranks=8, rank=0) as buffer:
+        x, idx, weights = (item.cuda() for item in inputs[0])
+        a = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        for round_index in range(3):
+            print(f"case: dispatch T={tokens} under concurrent GEMMs, round {round_index}", flush=True)
+            arm(buffer, inputs)
+            # GEMMs already occupy the GPU when the dispatch kernels are launched (a
+            # side stream the dispatch is not ordered after) ...
+            with torch.cuda.stream(side):
+                c = a
+                for _ in range(20):
+                    c = (a @ c).clamp_(-1, 1)
+            result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+            # ... and more arrive on the caller's stream while it runs (~1 TFLOP each).
+            b = a
+            for _ in range(40):
+                b = (a @ b).clamp_(-1, 1)
+            verify_dispatch(result, inputs, 0, WORLD, 256, 8, True, 1, False)
+            assert torch.isfinite(c.float().sum())
+            buffer.peers.wait(30_000)
+            assert torch.isfinite(b.float().sum())
+            del result
