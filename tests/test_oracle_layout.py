@@ -229,3 +229,42 @@ def test_cpu_baseline_matches_oracle(alignment, fp8):
             assert torch.equal(out["recv_x"][row].view(torch.int16), want[0].view(torch.int16))
             assert out["recv_weights"][row] == all_w[source][token, branch]
         assert not torch.count_nonzero(out["recv_x"][torch.from_numpy(e.padding_rows)].view(torch.int16))
+
+
+def test_cpu_plumbing_configuration_all_eight_receivers():
+    """The CPU-runnable configuration: 8 logical ranks in one process, T=64 tokens
+    per rank, hidden 512 BF16 ~ N(0,1), 16 experts (2 per rank), top-2 without
+    replacement, softmax weights, BF16 wire, expanded output.  Checked through
+    properties that hold for the dispatch as a whole: every routed branch lands
+    exactly once, on the rank that owns its expert, in its expert's segment, in
+    (source, token) order, carrying its source row."""
+    world, tokens, hidden, experts, topk = 8, 64, 512, 16, 2
+    generator = torch.Generator().manual_seed(20261024)
+    x = [torch.randn(tokens, hidden, generator=generator).to(torch.bfloat16) for _ in range(world)]
+    idx = [torch.rand(tokens, experts, generator=generator).topk(topk, dim=1).indices.numpy().astype(np.int64) for _ in range(world)]
+    bits = [item.view(torch.int16).numpy().view(np.uint16) for item in x]
+    local = experts // world
+    seen = set()
+    total_unique = 0
+    for rank in range(world):
+        expectation = oracle.expected_dispatch(idx, rank, world, experts, alignment=1)
+        receiver, rows = expectation.receiver, expectation.expanded
+        payload, valid = oracle.gather_expanded_payload(bits, rows)
+        assert receiver.expanded_count == rows.rows.size == int(receiver.expert_counts.sum()) == int(valid.sum())
+        assert receiver.expert_offsets.tolist() == np.concatenate([[0], np.cumsum(receiver.expert_counts)]).tolist()
+        # Expert-major, then source, then token: the row order is strictly increasing in that key.
+        key = (rows.expert.astype(np.int64) * world + rows.source) * tokens + rows.token
+        assert np.all(np.diff(key[np.argsort(rows.rows)]) > 0)
+        for row, source, token, branch, expert in zip(rows.rows, rows.source, rows.token, rows.branch, rows.expert):
+            assert idx[source][token, branch] == rank * local + expert
+            assert receiver.expert_offsets[expert] <= row < receiver.expert_offsets[expert] + receiver.expert_counts[expert]
+            assert np.array_equal(payload[row], bits[source][token])
+            assert (source, token, branch) not in seen
+            seen.add((source, token, branch))
+        # Unique rows: one per (source, token) with at least one expert on this rank.
+        hits = sum(int(np.any(idx[source] // local == rank, axis=1).sum()) for source in range(world))
+        assert receiver.unique_count == hits == int(receiver.source_offsets[-1])
+        total_unique += hits
+    assert len(seen) == world * tokens * topk  # nothing lost, nothing duplicated
+    volume = oracle.route_volume(idx, world, experts)
+    assert total_unique == volume["remote_deliveries"] + sum(int(np.any(idx[r] // local == r, axis=1).sum()) for r in range(world))
