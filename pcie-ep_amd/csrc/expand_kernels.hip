@@ -143,19 +143,21 @@ __global__ void __launch_bounds__(256) host_copy_kernel(char* host, u32x4* devic
     }
 }
 
-int row_grid(int64_t rows) {
+int row_grid(int64_t rows, int64_t cap = 8192) {
     // Four wavefronts per workgroup, one row per wavefront, capped so that the
     // grid-stride loop still spreads over all 256 CUs several times.
     int64_t blocks = (rows + 3) / 4;
     if (blocks < 1) blocks = 1;
-    if (blocks > 8192) blocks = 8192;
+    if (blocks > cap) blocks = cap;
     return int(blocks);
 }
 
 }  // namespace
 
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
-    const dim3 grid(row_grid(unique_capacity(state.z.dims))), block(256);
+    // One wavefront per possible unique row up to 65 536 rows (measured: a few
+    // percent faster than a grid-stride loop over fewer wavefronts).
+    const dim3 grid(row_grid(unique_capacity(state.z.dims), 16384)), block(256);
     if (state.z.dims.hidden % 8 == 0) hipLaunchKernelGGL(expand_kernel<true>, grid, block, 0, stream, state);
     else hipLaunchKernelGGL(expand_kernel<false>, grid, block, 0, stream, state);
     return hipGetLastError();
