@@ -10,7 +10,7 @@ GPU's own source are resident in HBM before the timed region; remote payloads
 are resident in pinned host memory, which is where this transport has them by
 definition.
 
-Prints ONE JSON line (metric of BASELINE.json: dispatch time and PCIe payload
+Prints ONE JSON line (the headline metric: dispatch time and PCIe payload
 rate against the measured pinned-copy peak, T=8192, H=7168, top-8) with
 ``roofline`` (stand-alone expand kernel against HBM), ``pcie`` (the transport
 kernel against the measured pinned hipMemcpy peak) and ``cpu_baseline`` (the
