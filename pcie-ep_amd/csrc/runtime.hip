@@ -140,6 +140,22 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     for (const void* pointer : required)
         if (!pointer) return set_error(PCIE_EP_E_INVALID, "an output pool pointer is NULL");
     if (a->expanded_capacity_rows <= 0) return set_error(PCIE_EP_E_INVALID, "expanded capacity must be positive");
+    // The kernels move rows as 16-byte vectors when the row length allows it and
+    // use 8-byte accesses for the 64-bit outputs: refuse pointers they would fault on.
+    auto misaligned = [](const void* pointer, uintptr_t alignment) { return pointer && reinterpret_cast<uintptr_t>(pointer) % alignment != 0; };
+    const uintptr_t row_alignment = d.hidden % 8 == 0 ? 16 : 2;
+    if (misaligned(a->x, row_alignment) || misaligned(a->unique_payload, row_alignment) || misaligned(a->expanded_payload, row_alignment))
+        return set_error(PCIE_EP_E_INVALID, "payload pointers must be %d-byte aligned for hidden=%d", int(row_alignment), d.hidden);
+    const void* words64[] = {a->topk_idx, a->unique_topk_idx, a->unique_source_meta, a->expanded_expert_idx, a->expanded_source_meta,
+                             a->unique_count, a->expanded_count, a->errors, a->stats, a->transport_timestamps_ns, a->channel_stats,
+                             a->channel_timestamps_ns, a->receive_expand_overlap, a->receive_prefix_state, a->prefix_tx_timestamps_ns};
+    for (const void* pointer : words64)
+        if (misaligned(pointer, 8)) return set_error(PCIE_EP_E_INVALID, "a 64-bit array pointer is not 8-byte aligned");
+    const void* words32[] = {a->topk_weights, a->unique_topk_weights, a->unique_expert_ordinals, a->expanded_weights, a->expert_prefix,
+                             a->expert_counts, a->expert_offsets, a->source_offsets, a->source_expert_prefix, a->expected_receive_counts};
+    for (const void* pointer : words32)
+        if (misaligned(pointer, 4)) return set_error(PCIE_EP_E_INVALID, "a 32-bit array pointer is not 4-byte aligned");
+    if (misaligned(a->plan, 256)) return set_error(PCIE_EP_E_INVALID, "route plan storage must be 256-byte aligned");
 
     std::memset(&s, 0, sizeof s);
     s.z = rt->z;

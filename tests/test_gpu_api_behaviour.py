@@ -226,3 +226,17 @@ def test_dispatch_overlaps_with_compute_on_another_stream():
             buffer.peers.wait(30_000)
             assert torch.isfinite(b.float().sum())
             del result
+
+
+def test_misaligned_payload_is_refused_by_the_native_boundary(inputs):
+    """Rows move as 16-byte vectors: a contiguous tensor whose storage offset breaks
+    that alignment must be rejected on the host, never handed to a kernel."""
+    with make_buffer(tmax=TOKENS, hidden=HIDDEN, channels=2) as buffer:
+        x, idx, weights = (item.cuda() for item in inputs[0])
+        shifted = torch.empty(x.numel() + 1, dtype=torch.bfloat16, device="cuda")[1:].view_as(x)
+        shifted.copy_(x)
+        assert shifted.is_contiguous() and shifted.data_ptr() % 16 == 2
+        with pytest.raises(RuntimeError, match="16-byte aligned"):
+            buffer.dispatch(shifted, idx, weights, do_expand=True)
+        result, _ = run_dispatch(buffer, inputs)  # the refusal consumed nothing
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
