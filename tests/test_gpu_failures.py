@@ -136,3 +136,13 @@ def test_delay_hooks_do_not_change_results(inputs):
         buffer.runtime.set_test_prefix_delay_ns(200_000)
         result, _ = run_dispatch(buffer, inputs)
         verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
+
+
+def test_expanded_capacity_overflow_is_code_16(inputs):
+    """A caller that provides fewer expanded rows than the routing needs gets a
+    terminal error, not an out-of-bounds write (the capacity formula of the
+    Python layer makes this unreachable there, so the limit is lowered by hand)."""
+    with small_buffer(timeout_ms=2000) as buffer:
+        print("case: expanded capacity lowered to 3 rows", flush=True)
+        buffer.runtime.sizes.expanded_rows = 3
+        failing_dispatch(buffer, inputs, 16)
