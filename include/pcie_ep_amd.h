@@ -154,6 +154,11 @@ int pcie_ep_set_test_delays(pcie_ep_runtime* runtime, uint64_t metadata_ns, uint
 int pcie_ep_set_test_prefix_delay_ns(pcie_ep_runtime* runtime, uint64_t delay_ns);
 int pcie_ep_set_test_control_abort_after_ns(pcie_ep_runtime* runtime, uint64_t delay_ns);
 int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* runtime, int32_t source);
+/* Overwrite the device-side epoch counter (synchronises the device).  Only for
+ * testing epoch exhaustion (error 20 once the epoch would reach 2^32:
+ * csrc/kernels/host_staged/advanced_layout.cuh:44-48); no counterpart in the
+ * reference, which has no test of that path. */
+int pcie_ep_set_test_epoch(pcie_ep_runtime* runtime, uint64_t epoch);
 
 /* Replaces get_device_numa_node (advanced_shared_memory.hpp:120-131). */
 int pcie_ep_device_numa_node(int32_t device);

@@ -434,6 +434,13 @@ int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* rt, int32_t source)
     return 0;
 }
 
+int pcie_ep_set_test_epoch(pcie_ep_runtime* rt, uint64_t epoch) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(rt->epoch, &epoch, sizeof epoch, hipMemcpyHostToDevice));
+    return 0;
+}
+
 int pcie_ep_device_numa_node(int32_t device) {
     char bus_id[64] = {};
     if (hipDeviceGetPCIBusId(bus_id, sizeof bus_id, device) != hipSuccess) return -1;

@@ -62,6 +62,7 @@ _PROTOTYPES = {
     "pcie_ep_set_test_prefix_delay_ns": (C.c_int, [C.c_void_p, C.c_uint64]),
     "pcie_ep_set_test_control_abort_after_ns": (C.c_int, [C.c_void_p, C.c_uint64]),
     "pcie_ep_set_test_skip_counts_ack_source": (C.c_int, [C.c_void_p, C.c_int32]),
+    "pcie_ep_set_test_epoch": (C.c_int, [C.c_void_p, C.c_uint64]),
     "pcie_ep_device_numa_node": (C.c_int, [C.c_int32]),
     "pcie_ep_host_signal_store": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_uint64]),
     "pcie_ep_host_signal_load": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64)]),

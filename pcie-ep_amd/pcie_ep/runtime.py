@@ -215,6 +215,9 @@ class NativeRuntime:
     def set_test_skip_counts_ack_source(self, source: int) -> None:
         _native.check(self._lib.pcie_ep_set_test_skip_counts_ack_source(self._require(), source), invalid=RuntimeError)
 
+    def set_test_epoch(self, epoch: int) -> None:
+        _native.check(self._lib.pcie_ep_set_test_epoch(self._require(), epoch), invalid=RuntimeError)
+
     def host_signal_store(self, segment_rank: int, which: int, index: int, value: int) -> None:
         _native.check(self._lib.pcie_ep_host_signal_store(self._require(), segment_rank, which, index, value))
 

@@ -146,3 +146,15 @@ def test_expanded_capacity_overflow_is_code_16(inputs):
         print("case: expanded capacity lowered to 3 rows", flush=True)
         buffer.runtime.sizes.expanded_rows = 3
         failing_dispatch(buffer, inputs, 16)
+
+
+def test_epoch_exhaustion_is_code_20(inputs):
+    """Sequences carry the epoch in their upper 32 bits; a buffer whose epoch would
+    reach 2^32 stops with a terminal error instead of wrapping."""
+    with small_buffer(timeout_ms=2000) as buffer:
+        result, _ = run_dispatch(buffer, inputs)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
+        del result
+        print("case: epoch counter set to 2^32 - 1", flush=True)
+        buffer.runtime.set_test_epoch(2**32 - 1)
+        failing_dispatch(buffer, inputs, 20)
