@@ -55,7 +55,7 @@ typedef struct pcie_ep_config {
     int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
     int32_t device;             /* HIP device ordinal */
     int32_t worker_groups;      /* payload workgroups of the transport kernel, spread over the XCDs;
-                                   0 = default (48), -1 = none (control workgroups move the rows) */
+                                   0 = default (48; 64 on the FP8 wire), -1 = none (control workgroups move the rows) */
     int32_t reserved[6];
 } pcie_ep_config;
 

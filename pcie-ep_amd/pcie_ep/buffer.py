@@ -129,7 +129,7 @@ class HostStagedEPBuffer:
         (default: one per peer, at most 7); ``staging_numa_node`` binds the pinned
         rings to a NUMA node; ``worker_groups`` / ``tx_waves`` / ``rx_waves``
         shape the transport kernel (0 = defaults: 48 payload workgroups of 2 TX +
-        2 RX wavefronts, 4 RX on the FP8 wire; ``worker_groups=-1`` makes the
+        2 RX wavefronts; 64 of 2 TX + 4 RX on the FP8 wire; ``worker_groups=-1`` makes the
         per-channel control workgroups move the rows themselves).
         """
         if not torch.cuda.is_available():
