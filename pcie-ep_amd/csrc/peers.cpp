@@ -380,9 +380,7 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
                         state.pending_sequence[slot_index] = 0;
                     }
                     const int ordinal = state.sent[channel];
-                    if (ordinal >= descriptors &&
-                        acquire(&descriptor_at(z_, own, channel, me_, ordinal)->consumed) != sequence(epoch, ordinal - descriptors))
-                        break;
+                    if (!credit_covers(acquire(credit_at(z_, own, channel, me_)), epoch, ordinal, descriptors)) break;
                     const bool last = fault == kFaultWrongPayloadSequence && cursor + 1 == int(list.size());
                     publish_token(state, rank, epoch, channel, token, slot, ordinal, last);
                     ++state.sent[channel];
@@ -489,7 +487,7 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                 std::atomic_thread_fence(std::memory_order_seq_cst);
                 const bool last = state.receive_done + 1 == state.receive_total;
                 if (!(fault == kFaultWithholdLastAck && last)) release(ack_at(z_, gpu, channel, slot, rank), payload_sequence);
-                release(&descriptor->consumed, sequence(epoch, ordinal));
+                release(credit_at(z_, gpu, channel, rank), sequence(epoch, ordinal));
                 ++state.consumed[channel];
                 ++state.receive_done;
                 progressed = true;

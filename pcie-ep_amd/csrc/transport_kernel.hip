@@ -418,10 +418,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                 device_store_b32(ring, at + 12, uint32_t(channel));
                 device_store_b32(ring, at + 16, uint32_t(payload_sequence));
                 device_store_b32(ring, at + 20, uint32_t(payload_sequence >> 32));
-                // The descriptor is captured: return its credit (this also waits
-                // for the ticket body), then tag the entry complete.  The payload
-                // ACK and the ring entry are separate resources.
-                host_store_release(&descriptor->consumed, sequence(epoch, ordinal));
+                // The ticket body is complete before its tag.
+                wait_memory_ops();
                 device_store(q.rx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
                 pending = false;
             }
@@ -434,6 +432,11 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             backoff();
         }
         issued += __popcll(accepted);
+        // Every accepted entry is captured in a ticket: return the credits, one
+        // store per source for the whole run (entries are consumed in order).  The
+        // payload ACK and the ticket ring entry are separate resources.
+        if (member && ahead == 0 && run > 0 && !failed)
+            host_field_store(credit_at(z, state.seg[source], channel, me), sequence(epoch, consumed + run - 1));
         if (member) consumed += run;
     }
     // RX is finished when every ticket has been retired by a worker.
@@ -580,9 +583,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         bool stop = false;
         while (true) {
             if (!slot_ok) slot_ok = host_load(ack_at(z, own, channel, slot, lane)) == previous_sequence;
-            if (!credit_ok)
-                credit_ok = host_load(&descriptor_at(z, own, channel, lane, my_descriptor)->consumed) ==
-                            sequence(epoch, my_descriptor - descriptors);
+            if (!credit_ok) credit_ok = credit_covers(host_load(credit_at(z, own, channel, lane)), epoch, my_descriptor, descriptors);
             if (__all(slot_ok && credit_ok)) break;
             ++credit_miss;
             if (broadcast_first((aborted(q) || deadline.expired(state)) ? 1 : 0)) {

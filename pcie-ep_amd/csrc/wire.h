@@ -4,7 +4,7 @@
 // One *segment* of pinned, fine-grained host memory exists per source rank.
 // Only the source writes payload slots, slot metadata, descriptor bodies,
 // READY words, the count mailbox, counts_ready, abort and channel_abort; a
-// receiver d writes only ack[..][d], the consumed word of its own (s -> d)
+// receiver d writes only ack[..][d], the credit word of its own (s -> d)
 // descriptor queue and counts_consumed[d].  Every 64-bit signal therefore has
 // exactly one writer and nothing ever performs a read-modify-write on host
 // memory (the discipline of the reference: csrc/kernels/host_staged/common.cuh:59-64).
@@ -72,26 +72,29 @@ struct alignas(128) Signal {
     char pad[120];
 };
 
-// One entry of a (source -> destination, channel) notification queue.  The
-// first 16 bytes are written by the source with ONE 16-byte store (the GPU) or
-// as fields followed by a release store of `ready` (a CPU), and read by the
-// destination with ONE 16-byte load (the GPU) or an acquire load of `ready`
-// followed by the fields (a CPU): a naturally aligned 16-byte access inside one
-// cache line is a single PCIe transaction and a single coherent snapshot, so
-// `payload_slot` and `token_index` are valid whenever `ready` matches.  The
-// payload sequence of the reference's descriptor is sequence(epoch,
-// token_index) by construction and is not stored separately; the destination's
-// unique-row ordinal travels in the slot metadata.  The destination alone
-// writes `consumed`.
-struct alignas(128) Descriptor {
+// One entry of a (source -> destination, channel) notification queue: 16 bytes,
+// written only by the source — with ONE 16-byte store (the GPU) or as fields
+// followed by a release store of `ready` (a CPU) — and read by the destination
+// with ONE 16-byte load (the GPU) or an acquire load of `ready` followed by the
+// fields (a CPU).  A naturally aligned 16-byte access inside one cache line is a
+// single PCIe transaction and a single coherent snapshot, so `payload_slot` and
+// `token_index` are valid whenever `ready` matches.  Entries are packed eight to
+// a 128-byte line, which is what one look-ahead poll of the GPU fetches.
+// The payload sequence of the reference's descriptor is sequence(epoch,
+// token_index) by construction and is not stored; the destination's unique-row
+// ordinal travels in the slot metadata.
+//
+// Credits flow the other way through ONE word per queue, written only by the
+// destination: sequence(epoch, last consumed ordinal).  Entries of a queue are
+// consumed in order, so the word says how many entries of this epoch are free
+// again (the reference keeps a consumed_sequence in every descriptor, which
+// puts two writers on one line).
+struct alignas(16) Descriptor {
     uint64_t ready;  // sequence(epoch, ordinal) once the entry is complete
     int32_t payload_slot;
     int32_t token_index;
-    uint64_t reserved[2];
-    uint64_t consumed;  // sequence(epoch, ordinal): credit returned by the destination
-    char pad[88];
 };
-static_assert(sizeof(Signal) == 128 && sizeof(Descriptor) == 128, "wire ABI");
+static_assert(sizeof(Signal) == 128 && sizeof(Descriptor) == 16, "wire ABI");
 
 // Per-slot token metadata, stored after the payload bytes of the slot.
 //   header (32 B) | rank_ordinals[kMaxRanks] (64 B) | expert_indices[K] |
@@ -140,7 +143,9 @@ struct SegmentLayout {
     size_t mailbox_offset;          // [P] blocks
     size_t slots_offset;            // [C*Q] slots, page aligned
     size_t ack_offset;              // [C*Q][P] signals
-    size_t descriptors_offset;      // [C][P][L] descriptors
+    size_t descriptors_offset;      // [C][P] queues of L packed entries, each queue 128-byte aligned
+    size_t descriptor_queue_stride;
+    size_t credits_offset;          // [C][P] signals: sequence(epoch, last ordinal the destination consumed)
     size_t size_bytes;
 };
 
@@ -172,7 +177,9 @@ PCIE_EP_HD SegmentLayout make_segment_layout(const Dimensions& dims) {
     const size_t slots = size_t(dims.channels) * dims.payload_slots;
     z.slots_offset = reserve(slots * z.slot_stride);
     z.ack_offset = reserve(slots * dims.num_ranks * sizeof(Signal));
-    z.descriptors_offset = reserve(size_t(dims.channels) * dims.num_ranks * dims.descriptor_slots * sizeof(Descriptor));
+    z.descriptor_queue_stride = align_up(size_t(dims.descriptor_slots) * sizeof(Descriptor), kSignalBytes);
+    z.descriptors_offset = reserve(size_t(dims.channels) * dims.num_ranks * z.descriptor_queue_stride);
+    z.credits_offset = reserve(size_t(dims.channels) * dims.num_ranks * sizeof(Signal));
     z.size_bytes = align_up(cursor, kPageBytes);
     return z;
 }
@@ -187,8 +194,18 @@ PCIE_EP_HD uint64_t* ack_at(const SegmentLayout& z, char* segment, int channel, 
     return signal_at(segment, z.ack_offset, (size_t(channel) * z.dims.payload_slots + slot) * z.dims.num_ranks + destination);
 }
 PCIE_EP_HD Descriptor* descriptor_at(const SegmentLayout& z, char* segment, int channel, int destination, int ordinal) {
-    return reinterpret_cast<Descriptor*>(segment + z.descriptors_offset) +
-        (size_t(channel) * z.dims.num_ranks + destination) * z.dims.descriptor_slots + ordinal % z.dims.descriptor_slots;
+    char* queue = segment + z.descriptors_offset + (size_t(channel) * z.dims.num_ranks + destination) * z.descriptor_queue_stride;
+    return reinterpret_cast<Descriptor*>(queue) + ordinal % z.dims.descriptor_slots;
+}
+PCIE_EP_HD uint64_t* credit_at(const SegmentLayout& z, char* segment, int channel, int destination) {
+    return signal_at(segment, z.credits_offset, size_t(channel) * z.dims.num_ranks + destination);
+}
+// The source may write entry `ordinal` of a queue of L entries once entry
+// `ordinal - L` has been consumed, i.e. once the credit word of this epoch
+// names an ordinal >= ordinal - L.
+PCIE_EP_HD bool credit_covers(uint64_t credit, uint64_t epoch, int ordinal, int descriptor_slots) {
+    if (ordinal < descriptor_slots) return true;
+    return (credit >> 32) == epoch && int64_t(credit & 0xFFFFFFFFull) - 1 >= int64_t(ordinal) - descriptor_slots;
 }
 PCIE_EP_HD int32_t* mailbox_at(const SegmentLayout& z, char* segment, int destination) {
     return reinterpret_cast<int32_t*>(segment + z.mailbox_offset + size_t(destination) * z.mailbox_stride);
