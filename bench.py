@@ -333,11 +333,12 @@ def main() -> int:
     mean = lambda values: sum(values) / len(values)
     transport_ms = mean(kernel_ms["transport"])
     dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"])
-    # Per remote row read: payload + slot metadata + one 16-byte descriptor poll;
-    # per own token written: payload + slot metadata, one 16-byte descriptor per
-    # destination; per remote row: an 8-byte payload ACK and an 8-byte credit.
+    # Per remote row read: payload + slot metadata + one 16-byte descriptor entry;
+    # per own token written: payload + slot metadata, one 16-byte descriptor entry
+    # per destination; per remote row: an 8-byte payload ACK, and an 8-byte credit
+    # for every polled run of up to eight entries.
     read_bytes = remote_reads * (payload_bytes + meta_bytes + 16)
-    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 16 + remote_reads * 16
+    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 16 + remote_reads * 9
     peak = max(h2d.value, d2h.value)
     step_s = ms_per_step * 1e-3
     value = (own_writes + remote_reads) * payload_bytes / step_s / 1e9
