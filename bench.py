@@ -4,17 +4,24 @@
 
 One step is one full dispatch of the receiver's share: the GPU is logical rank
 0 of 8; its own T tokens go through the real TX path into the pinned host ring,
-the 7 other sources are pre-staged by host threads in the same rings and are
-read once over PCIe and expanded into expert-major rows in HBM.  Inputs of the
-GPU's own source are resident in HBM before the timed region; remote payloads
-are resident in pinned host memory, which is where this transport has them by
-definition.
+the 7 other sources are staged by host threads in the same rings and are read
+once over PCIe and expanded into expert-major rows in HBM.  Inputs of the GPU's
+own source are resident in HBM before the timed region; remote payloads are
+resident in pinned host memory, which is where this transport has them by
+definition (the host threads do not rewrite unchanged rows between the timed
+steps: ``config.peer_restage`` is false; the ``restaged`` record repeats the
+measurement with every slot rewritten and every sent row read back per step).
 
-Prints ONE JSON line (the headline metric: dispatch time and PCIe payload
-rate against the measured pinned-copy peak, T=8192, H=7168, top-8) with
-``roofline`` (stand-alone expand kernel against HBM), ``pcie`` (the transport
-kernel against the measured pinned hipMemcpy peak) and ``cpu_baseline`` (the
-reference semantics of layout+expand in PyTorch on the host cores).
+Prints ONE JSON line.  Top level: the headline workload (dispatch time and PCIe
+payload rate against the measured pinned-copy peak, T=8192, H=7168, top-8, BF16
+wire) with ``roofline`` (stand-alone expand kernel against HBM), ``pcie`` (the
+transport kernel against the pinned hipMemcpy peak of the same run) and
+``cpu_baseline`` (layout + expand in PyTorch on the host cores).  The default run
+adds one compact record per further workload of the metric — ``fp8`` (FP8 wire,
+heavy-tailed inputs), ``hotspot_top4``, ``t4096``, ``eager_small_t``
+(T in 16..2048) and ``graph_replay_us`` (cached layout + hipGraph replay) —
+each timed the same way and each with a ``parity`` flag from an untimed
+dispatch checked bit for bit against the oracle.
 """
 
 from __future__ import annotations
@@ -35,6 +42,7 @@ WORLD, EXPERTS, HIDDEN = 8, 256, 7168
 HBM_PEAK_GBPS = 8000.0
 COPY_BYTES = 1 << 30  # calibration copy: 1 GiB read + 1 GiB written
 HOST_COPY_BYTES = 1 << 29  # kernel-driven pinned copy: 512 MiB each way
+BIT_EXACT = "bit-exact vs oracle"
 
 
 def log(*items) -> None:
@@ -47,11 +55,12 @@ def build_inputs(tokens: int, topk: int, routing: str, heavy_tail: bool):
     return baseline_inputs(tokens, topk, routing, heavy_tail, WORLD, EXPERTS, HIDDEN)
 
 
-def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000):
+def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000, graph=False):
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config = HostStagedConfig(channels=channels, stage=7 if wire == "fp8" else 6, wire_dtype="fp8_e4m3" if wire == "fp8" else "bf16",
-                              fuse_receive_expand=fuse, receive_expand_mode="pipelined" if fuse else "scalar", timeout_ms=timeout_ms)
+                              fuse_receive_expand=fuse, receive_expand_mode="pipelined" if fuse else "scalar", timeout_ms=timeout_ms,
+                              enable_graph=graph)
     return HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
                               num_ranks=WORLD, rank=0)
 
@@ -180,23 +189,125 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
         buffer.close()
 
 
-def graph_replay_sweep(topk, channels, sizes=(128, 512, 2048, 8192), replays=20):
-    """Cached layout + hipGraph replay: the plan is built by one eager dispatch,
-    the dispatch is captured with that plan, and `replays` GPU-only replays are
-    timed back to back (mean microseconds per replay, by size)."""
+def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, verify=True, restage=False):
+    """`steps` eager dispatches submitted back to back (wall clock per step), a second
+    pass with HIP events around every kernel, and one untimed dispatch checked
+    against the oracle.  Returns the measurements of this workload."""
     import torch
 
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+    from helpers import verify_dispatch
+
+    buffer = make_buffer(tokens, topk, wire, channels, fuse=True)
+    try:
+        sizes = buffer.runtime.sizes
+        payload_bytes, meta_bytes = int(sizes.payload_bytes), int(sizes.meta_bytes)
+        set_peers(buffer, inputs)
+        x, idx, weights = (item.cuda() for item in inputs[0])
+        buffer.peers.start(warmup + 2 * steps + (1 if verify else 0), restage=restage, read_rows=restage)
+        buffer.peers.wait_staged(120_000)
+        for _ in range(warmup):
+            result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+            del result
+        torch.cuda.synchronize()
+        # Timed region: exactly `steps` dispatches submitted back to back, as a
+        # steady caller would (nothing is read back, the CPU never waits inside).
+        started = time.perf_counter()
+        for _ in range(steps):
+            result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+            del result
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - started) / steps * 1e3
+
+        # Per-kernel durations: a second pass with HIP events recorded on the launch
+        # stream around every kernel (reading them waits for that dispatch, so this
+        # pass is not the one that is timed as a whole).
+        buffer.runtime.set_kernel_timing(True)
+        kernel_ms = {"prologue": [], "transport": []}
+        inside_ns = []
+        for _ in range(steps):
+            result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+            stamps = result[3].transport_timestamps_ns
+            times = buffer.runtime.kernel_times_ms()
+            for name in kernel_ms:
+                kernel_ms[name].append(times[name])
+            inside_ns.append(stamps.clone())
+            del result, stamps
+        torch.cuda.synchronize()
+        buffer.runtime.set_kernel_timing(False)
+        inside_ns = [item.cpu().tolist() for item in inside_ns]
+
+        # One more, checked bit for bit against the oracle (untimed).
+        parity = "skipped"
+        result = None
+        if verify:
+            result = buffer.dispatch(x, idx, weights, do_expand=True)
+            torch.cuda.synchronize()
+        buffer.peers.wait(120_000)
+        if result is not None:
+            summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, topk, True, 1, False, fp8_wire=wire == "fp8")
+            parity = BIT_EXACT
+            stats, unique, expanded = summary["stats"], summary["unique"], summary["expanded"]
+        else:
+            probe = buffer._last_handle
+            stats = probe.stats.cpu().tolist()
+            unique, expanded = int(probe.unique_count.cpu()), int(probe.expanded_count.cpu())
+        del result
+    finally:
+        buffer.close()
+
+    mean = lambda values: sum(values) / len(values)
+    own_writes, remote_reads, descriptors = int(stats[0]), int(stats[1]), int(stats[7])
+    transport_ms = mean(kernel_ms["transport"])
+    # Per remote row read: payload + slot metadata + one 16-byte descriptor entry;
+    # per own token written: payload + slot metadata, one 16-byte descriptor entry
+    # per destination; per remote row: an 8-byte payload ACK, and an 8-byte credit
+    # for every polled run of up to eight entries.
+    read_bytes = remote_reads * (payload_bytes + meta_bytes + 16)
+    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 16 + remote_reads * 9
+    h2d, d2h, kernel_read, kernel_write = peaks
+    pcie = {
+        "bound": "pcie", "kernel": "transport_kernel", "avg_us": transport_ms * 1e3, "min_us": min(kernel_ms["transport"]) * 1e3,
+        "inside_kernel_us": mean([(end - begin) / 1e3 for begin, end in inside_ns]),
+        "read_GBps": read_bytes / (transport_ms * 1e-3) / 1e9, "write_GBps": write_bytes / (transport_ms * 1e-3) / 1e9,
+        "read_payload_GBps": remote_reads * payload_bytes / (transport_ms * 1e-3) / 1e9,
+        "peak_h2d_GBps": h2d, "peak_d2h_GBps": d2h, "kernel_copy_read_GBps": kernel_read, "kernel_copy_write_GBps": kernel_write,
+        "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d,
+        "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
+    }
+    return {
+        "ms_per_step": ms_per_step, "kernel_ms": kernel_ms, "pcie": pcie, "parity": parity, "payload_bytes": payload_bytes,
+        "value": (own_writes + remote_reads) * payload_bytes / (ms_per_step * 1e-3) / 1e9,
+        "rows": {"own_published": own_writes, "remote_unique": remote_reads, "local_unique": unique - remote_reads, "expanded": expanded},
+    }
+
+
+def compact(run, tokens, topk):
+    """The sub-record of one further workload."""
+    mean = lambda values: sum(values) / len(values)
+    return {
+        "dispatch_us": run["ms_per_step"] * 1e3, "transport_us": mean(run["kernel_ms"]["transport"]) * 1e3,
+        "prologue_us": mean(run["kernel_ms"]["prologue"]) * 1e3, "payload_GBps": run["value"],
+        "pcie": run["pcie"]["frac"], "read_GBps": run["pcie"]["read_GBps"], "rows": run["rows"], "parity": run["parity"],
+        "logical_GBps": tokens * topk * HIDDEN * 2 / (run["ms_per_step"] * 1e-3) / 1e9,
+    }
+
+
+def graph_replay_sweep(topk, channels, sizes=(16, 128, 512, 2048, 8192), replays=20, inputs_by_size=None):
+    """Cached layout + hipGraph replay: the plan is built by one eager dispatch,
+    the dispatch is captured with that plan, `replays` GPU-only replays are
+    timed back to back (mean microseconds per replay, by size), and one more,
+    untimed, is checked against the oracle."""
+    import torch
+
+    from helpers import verify_dispatch
 
     out = {}
     for tokens in sizes:
-        inputs = build_inputs(tokens, topk, "uniform", False)
-        config = HostStagedConfig(channels=channels, enable_graph=True, timeout_ms=30000)
-        with HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
-                                num_ranks=WORLD, rank=0) as buffer:
+        inputs = (inputs_by_size or {}).get(tokens) or build_inputs(tokens, topk, "uniform", False)
+        with make_buffer(tokens, topk, "bf16", channels, fuse=True, graph=True) as buffer:
             set_peers(buffer, inputs)
             x, idx, weights = (item.cuda() for item in inputs[0])
-            buffer.peers.start(1 + 3 + replays)
+            buffer.peers.start(1 + 3 + replays + 1)
             result = buffer.dispatch(x, idx, weights, do_expand=True)
             cache = buffer.cache_layout(result[3])
             del result
@@ -208,12 +319,14 @@ def graph_replay_sweep(topk, channels, sizes=(128, 512, 2048, 8192), replays=20)
             for _ in range(replays):
                 graph.replay(async_with_compute_stream=True)
             torch.cuda.synchronize()
-            out[str(tokens)] = (time.perf_counter() - started) / replays * 1e6
+            replay_us = (time.perf_counter() - started) / replays * 1e6
+            result = graph.replay()
+            torch.cuda.synchronize()
             buffer.peers.wait(120_000)
-            error = buffer._last_handle.error.cpu().tolist()
-            if any(error):
-                raise RuntimeError(f"graph replay failed at T={tokens}: {error}")
-        log(f"[bench] graph replay T={tokens}: {out[str(tokens)]:.1f} us")
+            verify_dispatch(result, inputs, 0, WORLD, EXPERTS, topk, True, 1, False)
+            del result
+            out[str(tokens)] = {"replay_us": replay_us, "parity": BIT_EXACT}
+        log(f"[bench] graph replay T={tokens}: {replay_us:.1f} us")
     return out
 
 
@@ -229,8 +342,9 @@ def main() -> int:
     parser.add_argument("--skip-cpu-baseline", action="store_true")
     parser.add_argument("--skip-expand", action="store_true")
     parser.add_argument("--skip-verify", action="store_true")
-    parser.add_argument("--graph-sweep", action="store_true",
-                        help="also time cached-layout hipGraph replays for T in {128, 512, 2048, 8192}")
+    parser.add_argument("--only-headline", action="store_true",
+                        help="time only the workload named by --tokens/--wire/--routing (no fp8 / hotspot / T=4096 / small-T / "
+                             "graph-replay / restaged sub-records); what the profiler runs use")
     parser.add_argument("--expand-only", action="store_true",
                         help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
     args = parser.parse_args()
@@ -241,7 +355,6 @@ def main() -> int:
 
     import torch
 
-    from helpers import verify_dispatch
     from pcie_ep import _native
 
     torch.cuda.set_device(0)
@@ -267,110 +380,32 @@ def main() -> int:
         record["hbm_copy_GBps"] = copy_rate.value
         print(json.dumps({"roofline": record}), flush=True)
         return 0
+    peaks = (h2d.value, d2h.value, kernel_read.value, kernel_write.value)
 
-    buffer = make_buffer(tokens, topk, args.wire, args.channels, fuse=True)
-    sizes = buffer.runtime.sizes
-    payload_bytes, meta_bytes = int(sizes.payload_bytes), int(sizes.meta_bytes)
-    set_peers(buffer, inputs)
-    x, idx, weights = (item.cuda() for item in inputs[0])
-    total = args.warmup + 2 * args.steps + (0 if args.skip_verify else 1)
-    buffer.peers.start(total)
-    buffer.peers.wait_staged(120_000)
-    log("[bench] peers staged; warming up")
-    for _ in range(args.warmup):
-        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
-        del result
-    torch.cuda.synchronize()
-    # Timed region: exactly `steps` dispatches submitted back to back, as a
-    # steady caller would (nothing is read back, the CPU never waits inside).
-    started = time.perf_counter()
-    for _ in range(args.steps):
-        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
-        del result
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
-    ms_per_step = elapsed / args.steps * 1e3
-
-    # Per-kernel durations: a second pass with HIP events recorded on the launch
-    # stream around every kernel (reading them waits for that dispatch, so this
-    # pass is not the one that is timed as a whole).
-    buffer.runtime.set_kernel_timing(True)
-    kernel_ms = {"prologue": [], "transport": []}
-    inside_ns = []
-    for _ in range(args.steps):
-        result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
-        stamps = result[3].transport_timestamps_ns
-        times = buffer.runtime.kernel_times_ms()
-        for name in kernel_ms:
-            kernel_ms[name].append(times[name])
-        inside_ns.append(stamps.clone())
-        del result, stamps
-    torch.cuda.synchronize()
-    buffer.runtime.set_kernel_timing(False)
-    inside_ns = [item.cpu().tolist() for item in inside_ns]
-
-    # One more, checked bit for bit against the oracle (untimed).
-    parity = "skipped"
-    result = None
-    if not args.skip_verify:
-        result = buffer.dispatch(x, idx, weights, do_expand=True)
-        torch.cuda.synchronize()
-    buffer.peers.wait(120_000)
-    if result is not None:
-        summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, topk, True, 1, False, fp8_wire=args.wire == "fp8")
-        parity = "bit-exact vs oracle"
-        stats = summary["stats"]
-        unique, expanded = summary["unique"], summary["expanded"]
-    else:
-        probe = buffer._last_handle
-        stats = probe.stats.cpu().tolist()
-        unique, expanded = int(probe.unique_count.cpu()), int(probe.expanded_count.cpu())
-    del result
-    own_writes, remote_reads, descriptors = int(stats[0]), int(stats[1]), int(stats[7])
-    local_unique = unique - remote_reads
-    buffer.close()
-
+    log("[bench] headline workload")
+    run = run_workload(inputs, tokens, topk, args.wire, args.channels, args.steps, args.warmup, peaks, verify=not args.skip_verify)
     mean = lambda values: sum(values) / len(values)
-    transport_ms = mean(kernel_ms["transport"])
-    dispatch_gpu_ms = transport_ms + mean(kernel_ms["prologue"])
-    # Per remote row read: payload + slot metadata + one 16-byte descriptor entry;
-    # per own token written: payload + slot metadata, one 16-byte descriptor entry
-    # per destination; per remote row: an 8-byte payload ACK, and an 8-byte credit
-    # for every polled run of up to eight entries.
-    read_bytes = remote_reads * (payload_bytes + meta_bytes + 16)
-    write_bytes = own_writes * (payload_bytes + meta_bytes) + descriptors * 16 + remote_reads * 9
-    peak = max(h2d.value, d2h.value)
-    step_s = ms_per_step * 1e-3
-    value = (own_writes + remote_reads) * payload_bytes / step_s / 1e9
-    pcie = {
-        "bound": "pcie", "kernel": "transport_kernel", "avg_us": transport_ms * 1e3, "min_us": min(kernel_ms["transport"]) * 1e3,
-        "inside_kernel_us": mean([(end - begin) / 1e3 for begin, end in inside_ns]),
-        "read_GBps": read_bytes / (transport_ms * 1e-3) / 1e9, "write_GBps": write_bytes / (transport_ms * 1e-3) / 1e9,
-        "read_payload_GBps": remote_reads * payload_bytes / (transport_ms * 1e-3) / 1e9,
-        "peak_h2d_GBps": h2d.value, "peak_d2h_GBps": d2h.value,
-        "kernel_copy_read_GBps": kernel_read.value, "kernel_copy_write_GBps": kernel_write.value,
-        "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d.value,
-        "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
-    }
+    ms_per_step, kernel_ms, pcie = run["ms_per_step"], run["kernel_ms"], run["pcie"]
     traffic = counted_host_traffic(tokens, topk, args.routing, args.wire)
     pcie["traffic_read"], pcie["traffic_write"] = traffic["read"], traffic["write"]
     record = {
         "metric": "dispatch PCIe payload GB/s ((U+F_r)*B/t) and us per dispatch, receiver rank 0 of 8",
-        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "value": run["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.wire == "bf16" else "fp8_e4m3 wire / bf16",
         "data": "synthetic",
         "config": {
             "workload": f"T={tokens}/source x 8 logical ranks, h{HIDDEN}, top-{topk} {args.routing}, {EXPERTS} experts (32 local), "
                         f"{args.wire} wire, C{args.channels}, Q=L=256, expand on, own TX + 7 host-staged sources",
             "tokens_per_rank": tokens, "hidden": HIDDEN, "topk": topk, "experts": EXPERTS, "channels": args.channels, "wire": args.wire,
+            "peer_restage": False,
         },
-        "dispatch_us": ms_per_step * 1e3, "dispatch_gpu_us": dispatch_gpu_ms * 1e3,
+        "dispatch_us": ms_per_step * 1e3, "dispatch_gpu_us": (mean(kernel_ms["transport"]) + mean(kernel_ms["prologue"])) * 1e3,
         "kernel_us": {name: mean(values) * 1e3 for name, values in kernel_ms.items()},
         "dispatch_gpu_us_p50_p95": percentiles([1e3 * sum(step) for step in zip(*kernel_ms.values())]),
         "pcie_pct_of_peak": 100.0 * pcie["frac"],
-        "logical_GBps": tokens * topk * HIDDEN * 2 / step_s / 1e9,
-        "rows": {"own_published": own_writes, "remote_unique": remote_reads, "local_unique": local_unique, "expanded": expanded},
-        "parity": parity,
+        "logical_GBps": tokens * topk * HIDDEN * 2 / (ms_per_step * 1e-3) / 1e9,
+        "rows": run["rows"],
+        "parity": run["parity"],
         "pcie": pcie,
     }
     if not args.skip_expand:
@@ -382,11 +417,39 @@ def main() -> int:
         record["roofline"] = None
     if not args.skip_cpu_baseline:
         log("[bench] timing the CPU baseline on the host cores")
-        record["cpu_baseline"] = cpu_baseline(inputs, payload_bytes, fp8=args.wire == "fp8")
+        record["cpu_baseline"] = cpu_baseline(inputs, run["payload_bytes"], fp8=args.wire == "fp8")
     else:
         record["cpu_baseline"] = None
-    if args.graph_sweep:
-        record["graph_replay_us"] = graph_replay_sweep(topk, args.channels)
+
+    if not args.only_headline:
+        steps, warmup = args.steps, args.warmup
+        # The same workload with the host threads rewriting every slot and reading
+        # every sent row in every step: host-memory traffic concurrent with the
+        # GPU's.  Seven host threads cannot stage 0.5 GB per step as fast as the GPU
+        # reads it, so this figure is bounded by the emulator, not by the link.
+        log("[bench] headline workload, peers restaging every step")
+        restaged = run_workload(inputs, tokens, topk, args.wire, args.channels, max(3, steps // 4), 2, peaks, verify=False, restage=True)
+        record["restaged"] = {"dispatch_us": restaged["ms_per_step"] * 1e3, "transport_us": mean(restaged["kernel_ms"]["transport"]) * 1e3,
+                              "pcie": restaged["pcie"]["frac"], "peer_restage": True,
+                              "note": "every source slot rewritten and every sent row read by the host threads per step; bounded by their staging rate"}
+        uniform_8192 = inputs if (tokens, args.routing, args.wire) == (8192, "uniform", "bf16") else None
+        del inputs
+        log("[bench] fp8 wire, heavy-tailed inputs, T=8192 top-8")
+        record["fp8"] = compact(run_workload(build_inputs(8192, 8, "uniform", True), 8192, 8, "fp8", args.channels, steps, warmup, peaks), 8192, 8)
+        log("[bench] hotspot top-4, T=8192")
+        record["hotspot_top4"] = compact(run_workload(build_inputs(8192, 4, "hotspot", False), 8192, 4, "bf16", args.channels, steps, warmup, peaks), 8192, 4)
+        log("[bench] uniform top-8, T=4096")
+        record["t4096"] = compact(run_workload(build_inputs(4096, 8, "uniform", False), 4096, 8, "bf16", args.channels, steps, warmup, peaks), 4096, 8)
+        small = {}
+        small_inputs = {}
+        for size in (16, 128, 512, 2048):
+            small_inputs[size] = build_inputs(size, 8, "uniform", False)
+            small[str(size)] = compact(run_workload(small_inputs[size], size, 8, "bf16", args.channels, steps, warmup, peaks), size, 8)
+            log(f"[bench] eager T={size}: {small[str(size)]['dispatch_us']:.1f} us per dispatch")
+        record["eager_small_t"] = small
+        if uniform_8192 is not None:
+            small_inputs[8192] = uniform_8192
+        record["graph_replay_us"] = graph_replay_sweep(8, args.channels, replays=steps, inputs_by_size=small_inputs)
     print(json.dumps(record), flush=True)
     return 0
 

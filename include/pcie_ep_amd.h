@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define PCIE_EP_ABI_VERSION 1
+#define PCIE_EP_ABI_VERSION 2
 
 #define PCIE_EP_E_INVALID (-1)   /* bad argument / unsupported dimensions (ValueError / RuntimeError) */
 #define PCIE_EP_E_HIP (-2)       /* a HIP runtime call failed */
@@ -56,7 +56,17 @@ typedef struct pcie_ep_config {
     int32_t device;             /* HIP device ordinal */
     int32_t worker_groups;      /* payload workgroups of the transport kernel, spread over the XCDs;
                                    0 = default (48; 64 on the FP8 wire), -1 = none (control workgroups move the rows) */
-    int32_t reserved[6];
+    int32_t receive_expand_mode;/* 0 pipelined, 1 vectorized, 2 scalar (pcie_ep/config.py:58-60): selects what the
+                                   receive_expand_overlap diagnostic holds, the rows are moved the same way */
+    int32_t numa_mode;          /* 0 direct; 1 relay: ranks on another NUMA domain are reached through host relay
+                                   workers and replica rings (csrc/comm/numa_relay.hpp) */
+    int32_t replica_slots;      /* R per (channel, NUMA domain), relay mode */
+    int32_t relay_workers_per_numa; /* host relay threads per NUMA domain, 1..channels */
+    int32_t relay_cpu_count;    /* entries of relay_cpus in use; 0 = any CPU the process may run on */
+    int32_t reserved[5];
+    int32_t rank_numa_nodes[16];/* physical NUMA node of every rank, -1 = unknown (one domain) */
+    int32_t relay_cpus[64];     /* CPUs the relay workers may be pinned to */
+    uint64_t relay_delay_ns;    /* test hook: delay before each relay copy */
 } pcie_ep_config;
 
 /* Capacities and byte sizes a caller needs to allocate pools
@@ -220,7 +230,12 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
  * advanced_dispatch.cuh:73).  tokens may be 0. */
 int pcie_ep_peer_set_source(pcie_ep_runtime* runtime, int32_t rank, const void* x_bf16, const int64_t* topk_idx,
                             const float* weights, int32_t tokens);
-/* Serve the next `epochs` dispatches. flags bit 0: capture rows received from the GPU. */
+/* Serve the next `epochs` dispatches.  flags: bit 0 capture the rows received
+ * from the GPU; bit 1 stage every source slot afresh in every epoch (by default
+ * a slot whose row did not change since it was last written is only
+ * re-announced, so repeated epochs of one workload cause no host-memory writes
+ * besides descriptors); bit 2 the emulated receivers read every byte of the
+ * rows the GPU sent (by default they read the slot metadata only). */
 int pcie_ep_peers_start(pcie_ep_runtime* runtime, int32_t epochs, uint32_t flags);
 /* Block until every emulated source has staged all it can for the first
  * pending epoch without GPU progress (used to pre-stage before timing). */
@@ -239,7 +254,9 @@ int pcie_ep_peer_captured_copy(pcie_ep_runtime* runtime, int32_t rank, int32_t* 
                                float* weights, uint32_t* destination_masks);
 /* Force a protocol failure from the host.  fault: 1 withhold counts_ready,
  * 2 withhold counts_consumed, 3 withhold the last payload ACK, 4 publish a
- * wrong payload sequence.  Applies to rank `rank` for the next started epochs;
+ * wrong payload sequence, 5 send a unique-row ordinal beyond the announced
+ * count, 6 send an expert ordinal beyond the announced count (4-6 on the last
+ * row of every channel).  Applies to rank `rank` for the next started epochs;
  * fault 0 clears. */
 int pcie_ep_peers_inject_fault(pcie_ep_runtime* runtime, int32_t rank, int32_t fault);
 

@@ -10,7 +10,6 @@
 namespace pcie_ep {
 
 constexpr int kWave = 64;
-constexpr uint64_t kTicksPerUs = 100;  // wall_clock64() runs at 100 MHz on gfx950
 constexpr uint64_t kPrefixFailed = ~uint64_t(0);
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -34,7 +33,8 @@ struct alignas(16) RxEntry {
     int32_t token;
     int32_t channel;
     uint64_t payload_sequence;
-    uint64_t reserved;
+    int32_t channel_ordinal;  // position among the channel's receive tickets of this dispatch
+    int32_t reserved;
 };
 struct alignas(16) TxEntry {
     int32_t token;
@@ -78,7 +78,9 @@ struct DeviceState {
     int zero_padding;
     int reuse_plan;
     int counts_ack_skip_source;
+    int overlap_diagnostic;  // fill receive_expand_overlap (count, completion watermark); 0 leaves it zero
     uint64_t timeout_ticks;
+    uint64_t clock_khz;  // rate of wall_clock64() on this device (hipDeviceAttributeWallClockRate)
     uint64_t* epoch;
 
     const uint16_t* x;
@@ -141,7 +143,11 @@ struct DeviceState {
 // ---- clocks and back-off ---------------------------------------------------
 
 __device__ __forceinline__ uint64_t now_ticks() { return wall_clock64(); }
-__device__ __forceinline__ int64_t ticks_to_ns(uint64_t ticks) { return int64_t(ticks * (1000 / kTicksPerUs)); }
+// ticks * 1e6 / kHz without overflowing on absolute clock values.
+__device__ __forceinline__ int64_t ticks_to_ns(const DeviceState& state, uint64_t ticks) {
+    const uint64_t khz = state.clock_khz;
+    return int64_t(ticks / khz * 1000000ull + ticks % khz * 1000000ull / khz);
+}
 __device__ __forceinline__ void backoff() { __builtin_amdgcn_s_sleep(8); }
 
 __device__ inline void test_delay(uint64_t ticks) {
@@ -344,7 +350,7 @@ struct HealthCheck {
     int member, members, scans;
     __device__ HealthCheck(const DeviceState& state, uint64_t begin, bool progress_wait = false, int member_ = 0, int members_ = 1)
         : start(begin), member(member_), members(members_), scans(0) {
-        const uint64_t cap = 1000 * kTicksPerUs;
+        const uint64_t cap = state.clock_khz;  // one millisecond
         const uint64_t eighth = state.timeout_ticks / 8;
         interval = eighth < cap ? eighth : cap;
         next_scan = begin + interval;

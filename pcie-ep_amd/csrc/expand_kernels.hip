@@ -20,7 +20,7 @@ namespace {
 // (+ 36 bytes of row metadata per expanded row).  The payload loads of a row
 // are issued before the (dependent) metadata loads that name its destinations.
 template <bool kVector>
-__global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
+__global__ void __launch_bounds__(kRowKernelThreads) expand_kernel(DeviceState state) {
     if (load_error_code(state)) return;
     const SegmentLayout& z = state.z;
     const int lane = threadIdx.x % kWave;
@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(256) expand_kernel(DeviceState state) {
 }
 
 template <bool kVector>
-__global__ void __launch_bounds__(256) quantize_kernel(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden) {
+__global__ void __launch_bounds__(kRowKernelThreads) quantize_kernel(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden) {
     const int lane = threadIdx.x % kWave;
     const int waves_per_block = blockDim.x / kWave;
     const int total_waves = gridDim.x * waves_per_block;
@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint16_t* x, uint8_
 }
 
 template <bool kVector>
-__global__ void __launch_bounds__(256) dequantize_kernel(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden) {
+__global__ void __launch_bounds__(kRowKernelThreads) dequantize_kernel(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden) {
     const int lane = threadIdx.x % kWave;
     const int waves_per_block = blockDim.x / kWave;
     const int total_waves = gridDim.x * waves_per_block;
@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const uint8_t* codes, c
 // moves 16 KiB: 16 x 16-byte vectors per lane).  It exists to calibrate
 // measurements: the practical HBM ceiling of a read+write stream, and the
 // scale of the memory traffic counters for a kernel whose traffic is known.
-__global__ void __launch_bounds__(256) hbm_copy_kernel(const u32x4* source, u32x4* destination, int64_t vectors) {
+__global__ void __launch_bounds__(kRowKernelThreads) hbm_copy_kernel(const u32x4* source, u32x4* destination, int64_t vectors) {
     const int lane = threadIdx.x % kWave;
     const int waves_per_block = blockDim.x / kWave;
     const int64_t total_waves = int64_t(gridDim.x) * waves_per_block;
@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(256) hbm_copy_kernel(const u32x4* source, u32x
 // what a kernel (as opposed to the copy engine behind hipMemcpy) can pull over
 // the host link, and the scale of the host-traffic counters.
 template <bool kToDevice>
-__global__ void __launch_bounds__(256) host_copy_kernel(char* host, u32x4* device, int64_t vectors) {
+__global__ void __launch_bounds__(kRowKernelThreads) host_copy_kernel(char* host, u32x4* device, int64_t vectors) {
     const int lane = threadIdx.x % kWave;
     const int waves_per_block = blockDim.x / kWave;
     const int64_t total_waves = int64_t(gridDim.x) * waves_per_block;
@@ -157,7 +157,7 @@ int row_grid(int64_t rows, int64_t cap = 8192) {
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
     // One wavefront per possible unique row up to 65 536 rows (measured: a few
     // percent faster than a grid-stride loop over fewer wavefronts).
-    const dim3 grid(row_grid(unique_capacity(state.z.dims), 16384)), block(256);
+    const dim3 grid(row_grid(unique_capacity(state.z.dims), 16384)), block(kRowKernelThreads);
     if (state.z.dims.hidden % 8 == 0) hipLaunchKernelGGL(expand_kernel<true>, grid, block, 0, stream, state);
     else hipLaunchKernelGGL(expand_kernel<false>, grid, block, 0, stream, state);
     return hipGetLastError();
@@ -166,7 +166,7 @@ hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
 hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream) {
     const int64_t vectors = bytes / 16;
     if (vectors <= 0) return hipSuccess;
-    const dim3 grid(row_grid((vectors + kPassItems * kWave - 1) / (kPassItems * kWave))), block(256);
+    const dim3 grid(row_grid((vectors + kPassItems * kWave - 1) / (kPassItems * kWave))), block(kRowKernelThreads);
     hipLaunchKernelGGL(hbm_copy_kernel, grid, block, 0, stream, static_cast<const u32x4*>(source), static_cast<u32x4*>(destination), vectors);
     return hipGetLastError();
 }
@@ -174,7 +174,7 @@ hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hip
 hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_device, int wavefronts, hipStream_t stream) {
     const int64_t vectors = bytes / 16;
     if (vectors <= 0) return hipSuccess;
-    const dim3 grid(wavefronts < 4 ? 1 : wavefronts / 4), block(256);
+    const dim3 grid(wavefronts < 4 ? 1 : wavefronts / 4), block(kRowKernelThreads);
     if (to_device) hipLaunchKernelGGL(host_copy_kernel<true>, grid, block, 0, stream, static_cast<char*>(host), static_cast<u32x4*>(device), vectors);
     else hipLaunchKernelGGL(host_copy_kernel<false>, grid, block, 0, stream, static_cast<char*>(host), static_cast<u32x4*>(device), vectors);
     return hipGetLastError();
@@ -182,7 +182,7 @@ hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_dev
 
 hipError_t launch_quantize(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden, hipStream_t stream) {
     if (tokens <= 0) return hipSuccess;
-    const dim3 grid(row_grid(tokens)), block(256);
+    const dim3 grid(row_grid(tokens)), block(kRowKernelThreads);
     if (hidden % 16 == 0) hipLaunchKernelGGL(quantize_kernel<true>, grid, block, 0, stream, x, codes, scales, tokens, hidden);
     else hipLaunchKernelGGL(quantize_kernel<false>, grid, block, 0, stream, x, codes, scales, tokens, hidden);
     return hipGetLastError();
@@ -190,7 +190,7 @@ hipError_t launch_quantize(const uint16_t* x, uint8_t* codes, float* scales, int
 
 hipError_t launch_dequantize(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden, hipStream_t stream) {
     if (tokens <= 0) return hipSuccess;
-    const dim3 grid(row_grid(tokens)), block(256);
+    const dim3 grid(row_grid(tokens)), block(kRowKernelThreads);
     if (hidden % 16 == 0) hipLaunchKernelGGL(dequantize_kernel<true>, grid, block, 0, stream, codes, scales, out, tokens, hidden);
     else hipLaunchKernelGGL(dequantize_kernel<false>, grid, block, 0, stream, codes, scales, out, tokens, hidden);
     return hipGetLastError();

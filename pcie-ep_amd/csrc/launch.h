@@ -20,6 +20,14 @@ constexpr int kMaxTxWaves = 4;
 constexpr int kMaxRxWaves = 6;
 constexpr int kMaxWorkerGroups = 1024;
 
+// Workgroup sizes.  Each constant is used twice: as the __launch_bounds__ of the
+// kernel and by its launcher, so a launch shape can never exceed what the kernel
+// was compiled for (a block larger than the bound fails at launch).
+constexpr int kRowKernelThreads = 256;       // expand, FP8 wire, copy and fill kernels: four wavefronts
+constexpr int kTransportMaxThreads = 768;    // 2 control + at most 10 payload wavefronts
+constexpr int kPrologueMaxThreads = 1024;    // 16 wavefronts per token chunk
+static_assert((2 + kMaxTxWaves + kMaxRxWaves) * kWave <= kTransportMaxThreads, "transport workgroup exceeds its launch bound");
+
 // Epoch begin + layout + count publication (one workgroup per chunk of tokens).
 // The layout scratch holds prologue_flag_bytes() of zero-initialised chunk
 // flags followed by the per-chunk records.

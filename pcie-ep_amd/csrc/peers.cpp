@@ -176,7 +176,7 @@ void PeerEmulator::cancel() {
 }
 
 int PeerEmulator::inject_fault(int rank, int fault) {
-    if (rank < 0 || rank >= z_.dims.num_ranks || rank == me_ || fault < 0 || fault > 4) return -1;
+    if (rank < 0 || rank >= z_.dims.num_ranks || rank == me_ || fault < 0 || fault > kFaultExpertOrdinalOutOfRange) return -1;
     ranks_[rank].fault.store(fault);
     return 0;
 }
@@ -248,7 +248,7 @@ bool PeerEmulator::serve_epoch(int index, uint64_t epoch, std::string& error) {
         }
         state.pending_slots.clear();
         state.receive_total = state.receive_done = 0;
-        if (flags_ & 1u) {
+        if (flags_ & kPeerCapture) {
             state.cap_tokens.clear(); state.cap_rank_ordinals.clear(); state.cap_expert_idx.clear();
             state.cap_expert_ordinals.clear(); state.cap_payload.clear(); state.cap_scales.clear();
             state.cap_weights.clear(); state.cap_masks.clear();
@@ -299,12 +299,15 @@ bool PeerEmulator::serve_epoch(int index, uint64_t epoch, std::string& error) {
     }
 }
 
-void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int channel, int token, int slot, int ordinal, bool wrong_sequence) {
+void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int channel, int token, int slot, int ordinal, int fault) {
     const int topk = z_.dims.topk, ranks = z_.dims.num_ranks, hidden = z_.dims.hidden;
     char* own = seg_[rank];
     char* base = slot_at(z_, own, channel, slot);
     const size_t slot_index = size_t(channel) * z_.dims.payload_slots + slot;
-    if (state.slot_generation[slot_index] != state.generation || state.slot_token[slot_index] != token) {
+    const bool falsify = fault == kFaultRankOrdinalOutOfRange || fault == kFaultExpertOrdinalOutOfRange;
+    // Rows that did not change since the slot was last written are left in place
+    // unless the caller asked for every epoch to be staged afresh.
+    if ((flags_ & kPeerRestage) || falsify || state.slot_generation[slot_index] != state.generation || state.slot_token[slot_index] != token) {
         float scale = 1.0f;
         const uint16_t* row = state.x.data() + size_t(token) * hidden;
         if (z_.dims.wire_fp8) host_quantize_fp8(row, reinterpret_cast<uint8_t*>(base), &scale, 1, hidden);
@@ -324,12 +327,20 @@ void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int chan
         std::memcpy(branch + 2 * topk, state.weights.data() + size_t(token) * topk, size_t(topk) * 4);
         state.slot_generation[slot_index] = state.generation;
         state.slot_token[slot_index] = token;
+        if (falsify) {
+            // Fault hooks: an ordinal outside the counts this source announced.
+            if (fault == kFaultRankOrdinalOutOfRange) rank_ordinals[me_] = state.counts[me_];
+            else
+                for (int k = 0; k < topk; ++k)
+                    if (branch[k] >= 0 && branch[k] / z_.local_experts == me_) branch[topk + k] = 1 << 20;
+            state.slot_token[slot_index] = -1;  // stage the true row again next time
+        }
     }
     Descriptor* descriptor = descriptor_at(z_, own, channel, me_, ordinal);
     descriptor->payload_slot = slot;
     // The token identifies the payload (its sequence is sequence(epoch, token));
     // the fault hook publishes a token that does not match the slot's metadata.
-    descriptor->token_index = wrong_sequence ? token + 1 : token;
+    descriptor->token_index = fault == kFaultWrongPayloadSequence ? token + 1 : token;
     release(&descriptor->ready, sequence(epoch, ordinal));
     state.pending_sequence[slot_index] = sequence(epoch, token);
     if (!state.pending_listed[slot_index]) {
@@ -381,8 +392,9 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
                     }
                     const int ordinal = state.sent[channel];
                     if (!credit_covers(acquire(credit_at(z_, own, channel, me_)), epoch, ordinal, descriptors)) break;
-                    const bool last = fault == kFaultWrongPayloadSequence && cursor + 1 == int(list.size());
-                    publish_token(state, rank, epoch, channel, token, slot, ordinal, last);
+                    // Row faults apply to the last row this source sends to the GPU on the channel.
+                    const bool last = state.sent[channel] + 1 == state.channel_counts[size_t(channel) * ranks + me_];
+                    publish_token(state, rank, epoch, channel, token, slot, ordinal, last ? fault : kFaultNone);
                     ++state.sent[channel];
                 }
                 // Tokens bound only for other emulated ranks need no transfer here:
@@ -470,7 +482,13 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                     error = "GPU sent a token to a rank outside its destination mask";
                     return false;
                 }
-                if (flags_ & 1u) {
+                if (flags_ & kPeerReadRows) {
+                    const uint64_t* words = reinterpret_cast<const uint64_t*>(base);
+                    uint64_t sum = 0;
+                    for (int i = 0; i < z_.payload_bytes / 8; ++i) sum += words[i];
+                    state.read_checksum += sum;
+                }
+                if (flags_ & kPeerCapture) {
                     const char* meta = base + z_.meta_offset;
                     const int32_t* branch = reinterpret_cast<const int32_t*>(meta + kMetaBranchOffset);
                     state.cap_tokens.push_back(token);

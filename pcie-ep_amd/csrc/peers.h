@@ -34,6 +34,15 @@ enum PeerFault : int {
     kFaultWithholdCountsConsumed = 2,
     kFaultWithholdLastAck = 3,
     kFaultWrongPayloadSequence = 4,
+    kFaultRankOrdinalOutOfRange = 5,    // last row: unique-row ordinal beyond the announced count
+    kFaultExpertOrdinalOutOfRange = 6,  // last row: expert ordinal beyond the announced count
+};
+
+// Flags of PeerEmulator::start.
+enum PeerFlag : uint32_t {
+    kPeerCapture = 1u,   // receivers keep a copy of every row the GPU sent
+    kPeerRestage = 2u,   // sources rewrite payload and metadata of every slot in every epoch
+    kPeerReadRows = 4u,  // receivers read every byte of the rows the GPU sent
 };
 
 class PeerEmulator {
@@ -82,6 +91,7 @@ private:
         std::vector<float> cap_scales, cap_weights;
         std::vector<uint32_t> cap_masks;
         std::atomic<int> fault{0};
+        uint64_t read_checksum = 0;  // sink of kPeerReadRows
         std::atomic<uint64_t> staged_epoch{0};
     };
 
@@ -89,7 +99,7 @@ private:
     bool serve_epoch(int index, uint64_t epoch, std::string& error);
     bool source_progress(int rank, uint64_t epoch, bool& done, bool& quiescent, std::string& error);
     bool receiver_progress(int rank, uint64_t epoch, bool& done, std::string& error);
-    void publish_token(Rank& state, int rank, uint64_t epoch, int channel, int token, int slot, int ordinal, bool wrong_sequence);
+    void publish_token(Rank& state, int rank, uint64_t epoch, int channel, int token, int slot, int ordinal, int fault);
     void fail(const std::string& message);
 
     SegmentLayout z_;

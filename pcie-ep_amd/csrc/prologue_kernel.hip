@@ -62,7 +62,7 @@ struct ChunkRecord {
 };
 
 template <int kTopk>
-__global__ void __launch_bounds__(1024) prologue_kernel(DeviceState state, int chunk_waves, int chunks) {
+__global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceState state, int chunk_waves, int chunks) {
     extern __shared__ __align__(16) unsigned char lds[];
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, experts = z.dims.num_experts, topk = z.dims.topk;
@@ -351,6 +351,7 @@ hipError_t launch_prologue(const DeviceState& state, hipStream_t stream) {
     if (bytes > 64 * 1024) return hipErrorInvalidValue;  // cannot happen within the supported dimensions
     // At least 256 threads so the clear / publish loops stay short.
     const int threads = waves * kWave < 256 ? 256 : waves * kWave;
+    if (threads > kPrologueMaxThreads) return hipErrorInvalidValue;
     const int chunks = state.reuse_plan ? 0 : prologue_chunks(state.z, state.num_tokens);
     const dim3 grid(chunks > 1 ? chunks : 1);
     if (narrow) hipLaunchKernelGGL(prologue_kernel<8>, grid, dim3(threads), bytes, stream, state, waves, chunks);

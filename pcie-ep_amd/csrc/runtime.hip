@@ -87,6 +87,9 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
         return set_error(PCIE_EP_E_INVALID, "tx_waves must be 0..%d and rx_waves 0..%d", kMaxTxWaves, kMaxRxWaves);
     if (c->worker_groups < -1 || c->worker_groups > kMaxWorkerGroups)
         return set_error(PCIE_EP_E_INVALID, "worker_groups must be -1..%d", kMaxWorkerGroups);
+    if (c->receive_expand_mode < 0 || c->receive_expand_mode > 2) return set_error(PCIE_EP_E_INVALID, "receive_expand_mode must be 0 (pipelined), 1 (vectorized) or 2 (scalar)");
+    // Row bytes, slot offsets and the prologue's token keys are 32-bit quantities.
+    if (c->hidden > (1 << 24) || c->max_tokens > (1 << 24)) return set_error(PCIE_EP_E_INVALID, "hidden and max_tokens must not exceed 2^24");
     if (c->peer_threads < 0) return set_error(PCIE_EP_E_INVALID, "peer_threads must be non-negative");
     if (c->staging_numa_node < -1 || c->staging_numa_node >= 1024) return set_error(PCIE_EP_E_INVALID, "staging_numa_node must be -1..1023");
     dims = Dimensions{c->num_ranks, c->max_tokens, c->hidden, c->topk, c->num_experts, c->channels, c->payload_slots, c->descriptor_slots,
@@ -126,7 +129,9 @@ struct pcie_ep_runtime {
     uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
     int counts_ack_skip_source = -1;
     std::unique_ptr<PeerEmulator> peers;
+    uint64_t clock_khz = 100000;  // wall clock of the device, queried at creation
     bool closed = false;
+    uint64_t ticks_of_ns(uint64_t ns) const { return ns / 1000000 * clock_khz + ns % 1000000 * clock_khz / 1000000; }
     // Optional per-kernel timing with HIP events on the launch stream.
     bool timing = false;
     bool timing_valid = false;
@@ -136,7 +141,7 @@ struct pcie_ep_runtime {
 
 namespace {
 
-uint64_t ns_to_ticks(uint64_t ns) { return ns / (1000 / kTicksPerUs); }
+
 
 int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState& s) {
     const Dimensions& d = rt->z.dims;
@@ -196,7 +201,9 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.zero_padding = a->zero_padding ? 1 : 0;
     s.reuse_plan = a->reuse_plan ? 1 : 0;
     s.counts_ack_skip_source = rt->counts_ack_skip_source;
-    s.timeout_ticks = uint64_t(rt->config.timeout_ms) * 1000 * kTicksPerUs;
+    s.overlap_diagnostic = s.fuse_expand && s.expand && rt->config.receive_expand_mode == 0;
+    s.timeout_ticks = uint64_t(rt->config.timeout_ms) * rt->clock_khz;
+    s.clock_khz = rt->clock_khz;
     s.epoch = rt->epoch;
     s.x = static_cast<const uint16_t*>(a->x);
     s.topk_idx = a->topk_idx;
@@ -291,6 +298,12 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     HIP_TRY(hipSetDevice(config->device));
     auto rt = std::make_unique<pcie_ep_runtime>();
     rt->config = *config;
+    // Every device-side timeout, back-off period and timestamp is derived from the
+    // rate of the constant wall clock the kernels read.
+    int clock_khz = 0;
+    HIP_TRY(hipDeviceGetAttribute(&clock_khz, hipDeviceAttributeWallClockRate, config->device));
+    if (clock_khz <= 0) return set_error(PCIE_EP_E_HIP, "device %d reports no wall clock rate", config->device);
+    rt->clock_khz = uint64_t(clock_khz);
     rt->z = make_segment_layout(dims);
     rt->plan = plan_layout(dims);
     const LaunchShape shape = resolve_launch_shape(*config);
@@ -428,20 +441,20 @@ int pcie_ep_expand_unique(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args
 
 int pcie_ep_set_test_delays(pcie_ep_runtime* rt, uint64_t metadata_ns, uint64_t tx_ns, uint64_t rx_ns, uint64_t scatter_ns) {
     if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
-    rt->metadata_delay = ns_to_ticks(metadata_ns);
-    rt->tx_delay = ns_to_ticks(tx_ns);
-    rt->rx_delay = ns_to_ticks(rx_ns);
-    rt->scatter_delay = ns_to_ticks(scatter_ns);
+    rt->metadata_delay = rt->ticks_of_ns(metadata_ns);
+    rt->tx_delay = rt->ticks_of_ns(tx_ns);
+    rt->rx_delay = rt->ticks_of_ns(rx_ns);
+    rt->scatter_delay = rt->ticks_of_ns(scatter_ns);
     return 0;
 }
 int pcie_ep_set_test_prefix_delay_ns(pcie_ep_runtime* rt, uint64_t delay_ns) {
     if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
-    rt->prefix_delay = ns_to_ticks(delay_ns);
+    rt->prefix_delay = rt->ticks_of_ns(delay_ns);
     return 0;
 }
 int pcie_ep_set_test_control_abort_after_ns(pcie_ep_runtime* rt, uint64_t delay_ns) {
     if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
-    rt->control_abort_after = ns_to_ticks(delay_ns);
+    rt->control_abort_after = rt->ticks_of_ns(delay_ns);
     return 0;
 }
 int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* rt, int32_t source) {

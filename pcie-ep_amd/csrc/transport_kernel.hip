@@ -119,7 +119,7 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     const uint64_t start = now_ticks();
     HealthCheck health(state, start);
     if (lane == 0) {
-        state.prefix_tx_timestamps_ns[0] = ticks_to_ns(start);
+        state.prefix_tx_timestamps_ns[0] = ticks_to_ns(state, start);
         test_delay(state.prefix_delay);
     }
     // All sources are polled in parallel, one lane each.
@@ -209,7 +209,7 @@ __device__ bool prepare_receive_prefixes(const DeviceState& state, int lane) {
         const bool success = compute_receive_prefixes(state, lane);
         __threadfence();
         if (lane == 0) {
-            state.prefix_tx_timestamps_ns[1] = ticks_to_ns(now_ticks());
+            state.prefix_tx_timestamps_ns[1] = ticks_to_ns(state, now_ticks());
             store_release_device(state.receive_prefix_state + 1, success ? epoch : kPrefixFailed);
         }
     }
@@ -240,7 +240,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
     HealthCheck health(state, start, true, channel, channels);
-    if (lane == 0) device_store(state.channel_timestamps_ns + channel * 2, ticks_to_ns(start));
+    if (lane == 0) device_store(state.channel_timestamps_ns + channel * 2, ticks_to_ns(state, start));
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;
     const uint64_t below = lanes_below(lane);
@@ -250,7 +250,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
 #pragma unroll
     for (int rank = 0; rank < kMaxRanks; ++rank) reserved[rank] = 0;
     bool failed = false;
-    int64_t stage_busy = 0;
+    int64_t stage_busy = 0, prepared_ahead = 0;
 
     for (int base = 0; base < candidates && !failed; base += kWave) {
         const int candidate = base + lane;
@@ -272,6 +272,10 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         // Ring history: which token occupied ordinal i (needed when a slot is reused).
         if (remote) device_store(state.chan_remote_tokens + size_t(channel) * stride + ordinal, token);
         const int ticket_index = reserve_tickets(q.tx_tail, __popcll(batch), lane) + __popcll(batch & below);
+        // Tickets prepared while an earlier payload of this channel is still in
+        // flight: the control path runs ahead of the payload path (the event the
+        // reference counts in stats[3]: advanced_dispatch.cuh:384-387).
+        if (produced > 0 && broadcast_first(int(device_load(&q.tx_retired[channel].value))) < produced) prepared_ahead += __popcll(batch);
         bool pending = remote != 0;
         while (true) {
             if (pending && ring_entry_free(q.tx_taken, epoch, ticket_index)) {
@@ -290,7 +294,14 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
             }
             if (!__any(pending)) break;
             ++stage_busy;
-            if (health.poll(state, lane) || broadcast_first(aborted(q) ? 1 : 0)) {
+            const bool unhealthy = health.poll(state, lane);
+            if (unhealthy || broadcast_first(aborted(q) ? 1 : 0)) {
+                // A peer's abort flag or the timeout: raise the kernel-wide abort at
+                // once, the workers are spinning on tickets that will never be marked ready.
+                if (unhealthy && lane == 0) {
+                    record_error(state, kErrRingProgressWait);
+                    raise_abort(q);
+                }
                 failed = true;
                 break;
             }
@@ -304,7 +315,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     // Lanes poll different (ordinal, destination) pairs in parallel.
     bool drained = failed;
     int drain_ordinal = produced > slots ? produced - slots : 0;
-    bool workers_finished = false, announced = false;
+    bool workers_finished = false;
     while (true) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
@@ -325,15 +336,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
             else drain_ordinal += __builtin_ctzll(missing) / ranks;  // everything before the first miss is done
             if (drain_ordinal >= produced) drained = true;
         }
-        if (workers_finished && drained) {
-            if (!announced) {
-                // Diagnostic: when this channel's transmit side was drained,
-                // relative to the channel's start (column 1; column 0 is RX).
-                if (lane == 0) state.receive_expand_overlap[channel * 2 + 1] = ticks_to_ns(now_ticks() - start);
-                announced = true;
-            }
-            if (broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
-        }
+        if (workers_finished && drained && broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
         // Guardian: this wavefront outlives TX so that a stalled RX still times out.
         const bool unhealthy = health.poll(state, lane);
         const bool forced = channel == 0 && state.control_abort_after && now_ticks() - start >= state.control_abort_after;
@@ -349,10 +352,12 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     if (lane == 0) {
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRingFull),
                   static_cast<unsigned long long>(stage_busy));
+        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatPreparedAhead),
+                  static_cast<unsigned long long>(prepared_ahead));
         // Only this wavefront writes the channel's mapped abort word.
         if (aborted(q)) store_release_system(signal_at(own, z.channel_abort_offset, channel), epoch);
         // Both directions are complete (or aborted): the channel's end time.
-        device_store(state.channel_timestamps_ns + channel * 2 + 1, ticks_to_ns(now_ticks()));
+        device_store(state.channel_timestamps_ns + channel * 2 + 1, ticks_to_ns(state, now_ticks()));
     }
 }
 
@@ -382,10 +387,9 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
     Deadline deadline(begin);
     int consumed = 0, issued = 0;
-    int64_t not_ready = 0, iterations = 0, ring_waits = 0;
+    int64_t not_ready = 0, ring_waits = 0;
     bool failed = false;
     while (issued < total && !failed) {
-        ++iterations;
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
@@ -418,6 +422,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                 device_store_b32(ring, at + 12, uint32_t(channel));
                 device_store_b32(ring, at + 16, uint32_t(payload_sequence));
                 device_store_b32(ring, at + 20, uint32_t(payload_sequence >> 32));
+                device_store_b32(ring, at + 24, uint32_t(issued + __popcll(accepted & below)));
                 // The ticket body is complete before its tag.
                 wait_memory_ops();
                 device_store(q.rx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
@@ -448,11 +453,9 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     if (lane == 0) {
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxNotReady),
                   static_cast<unsigned long long>(not_ready));
-        // Diagnostic: when this channel's receive side finished, relative to the
-        // channel's start (column 0), next to the transmit side's drain (column 1).
-        state.receive_expand_overlap[channel * 2] = ticks_to_ns(now_ticks() - begin);
-        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxPolls),
-                  static_cast<unsigned long long>(iterations));
+        // Column 1 of the receive/expand diagnostic: how many receive tickets of
+        // this channel have completed their scatter (fused_receive.cuh:290-294).
+        if (state.overlap_diagnostic) state.receive_expand_overlap[channel * 2 + 1] = int64_t(device_load(&q.rx_retired[channel].value));
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRingFull),
                   static_cast<unsigned long long>(ring_waits));
         device_store(&q.rx_finished[channel].value, 1u);
@@ -566,7 +569,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         if (lane == 0) device_store(q.tx_taken + ticket_index % kRing, sequence(epoch, ticket_index));
         const int slot = ordinal % slots;
         const bool targeted = lane < ranks && ((endpoints >> lane) & 1u);
-        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(now_ticks());
+        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(state, now_ticks());
 
         // Flow control: the slot's previous occupant must be ACKed by all its
         // targets and a descriptor entry must have been consumed before reuse
@@ -629,7 +632,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
             const u32x4 entry = {uint32_t(ready), uint32_t(ready >> 32), uint32_t(slot), uint32_t(token)};
             host_store_b128(host_resource(descriptor_at(z, own, channel, lane, my_descriptor), 16), 0, entry);
         }
-        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(now_ticks());
+        if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(state, now_ticks());
         ++writes;
         deliveries += __popc(endpoints);
         fence_lds();  // scratch is reused by the next ticket
@@ -667,6 +670,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         const int source = __shfl(int(word), 0), slot = __shfl(int(word), 1), ticket_token = __shfl(int(word), 2);
         const int channel = __shfl(int(word), 3);
         const uint64_t payload_sequence = uint64_t(uint32_t(__shfl(int(word), 4))) | uint64_t(uint32_t(__shfl(int(word), 5))) << 32;
+        const int channel_ordinal = __shfl(int(word), 6);
         // The ticket now lives in registers: its ring entry may be reused while
         // this wavefront is still moving the row.
         wait_memory_ops();
@@ -675,6 +679,12 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         const __amdgpu_buffer_rsrc_t payload = host_resource(slot_base, uint32_t(z.payload_bytes));
         const __amdgpu_buffer_rsrc_t slot_meta = host_resource(slot_base + z.meta_offset, uint32_t(z.meta_bytes));
         if (lane == kWave - 1) test_delay(state.rx_delay);
+        // Column 0 of the receive/expand diagnostic: this row's host read starts
+        // while an earlier row of the channel has not finished its scatter (the
+        // conservative proof point of fused_receive.cuh:216-225; a count, not a time).
+        if (state.overlap_diagnostic && lane == 0 && channel_ordinal > 0 &&
+            int(device_load(&q.rx_retired[channel].value)) < channel_ordinal)
+            atomicAdd(reinterpret_cast<unsigned long long*>(state.receive_expand_overlap + channel * 2), 1ull);
 
         // Metadata first (it arrives first), payload right behind it.
         const uint32_t meta_lo = host_load_b32(slot_meta, uint32_t(lane) * 4u);  // out of range reads as 0
@@ -708,21 +718,41 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
             break;
         }
 
-        // Destination rows, one lane per branch.
+        // Destination rows, one lane per branch.  Everything the row numbers are
+        // made of comes from the peer: the token must be addressed to this rank and
+        // its ordinals must lie inside the counts that peer announced, or a store
+        // would land in another expert's rows or before the pool.  Same verdict as a
+        // wrong identity: terminal, and the slot is not ACKed.
         int64_t my_row = -1;
         int my_expert = -1;
-        if (scatter) {
-            if (lane < topk) {
-                const int global_expert = int(scratch[kMetaBranchOffset / 4 + lane]);
-                const int expert = global_expert - me * local;
-                if (global_expert >= 0 && expert >= 0 && expert < local) {
+        bool out_of_range = lane == 0 && !((scratch[1] >> me) & 1u);
+        if (lane < topk) {
+            const int global_expert = int(scratch[kMetaBranchOffset / 4 + lane]);
+            const int expert = global_expert - me * local;
+            if (global_expert >= 0 && expert >= 0 && expert < local) {
+                const int ordinal = int(scratch[kMetaBranchOffset / 4 + topk + lane]);
+                const int before = device_load(state.source_expert_prefix + source * local + expert);
+                const int through = source + 1 < z.dims.num_ranks ? device_load(state.source_expert_prefix + (source + 1) * local + expert)
+                                                                  : device_load(state.expert_counts + expert);
+                out_of_range |= ordinal < 0 || ordinal >= through - before;
+                if (scatter) {
                     my_expert = expert;
-                    my_row = int64_t(device_load(state.expert_offsets + expert)) + device_load(state.source_expert_prefix + source * local + expert) +
-                             int(scratch[kMetaBranchOffset / 4 + topk + lane]);
+                    my_row = int64_t(device_load(state.expert_offsets + expert)) + before + ordinal;
                 }
             }
-        } else if (lane == 0) {
-            my_row = int64_t(device_load(state.source_offsets + source)) + int(scratch[kMetaRankOrdinalsOffset / 4 + me]);
+        }
+        if (lane == 0) {
+            const int ordinal = int(scratch[kMetaRankOrdinalsOffset / 4 + me]);
+            const int first = device_load(state.source_offsets + source);
+            out_of_range |= ordinal < 0 || ordinal >= device_load(state.source_offsets + source + 1) - first;
+            if (!scatter) my_row = int64_t(first) + ordinal;
+        }
+        if (__any(out_of_range)) {
+            if (lane == 0) {
+                record_error(state, kErrPayloadSequence);
+                raise_abort(q);
+            }
+            break;
         }
         const int64_t capacity = scatter ? state.expanded_capacity : unique_capacity(z.dims);
         if (__any(my_row >= capacity)) {
@@ -851,7 +881,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
 // no payload workgroups configured the control workgroups carry the payload
 // wavefronts themselves.
 template <bool kFp8, bool kVector>
-__global__ void __launch_bounds__(768) transport_kernel(DeviceState state) {
+__global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceState state) {
     __shared__ WaveScratch lds;
     const int channels = state.z.dims.channels;
     if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) return;
@@ -895,6 +925,7 @@ int transport_threads(const DeviceState& state) {
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
     const dim3 grid(state.z.dims.channels + (state.worker_groups > 0 ? state.worker_groups : 0) + state.local_groups), block(transport_threads(state));
+    if (int(block.x) > kTransportMaxThreads) return hipErrorInvalidValue;
     const bool fp8 = state.z.dims.wire_fp8 != 0;
     // BF16 rows need 16-byte granularity on both sides; FP8 additionally needs
     // whole 16-code vectors on the wire.

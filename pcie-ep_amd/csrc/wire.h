@@ -20,7 +20,7 @@
 #include <cstddef>
 #include <cstdint>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define PCIE_EP_HD __host__ __device__ inline
 #else
 #define PCIE_EP_HD inline
@@ -58,12 +58,11 @@ enum StatField : int {
     kStatHostWrites = 0,     // own tokens published to the host ring
     kStatHostReads = 1,      // remote unique rows read from host rings
     kStatDeliveries = 2,     // sum over published tokens of remote destination ranks
-    // 3..6 are event counters of this implementation (the reference leaves them
-    // implementation specific); they depend on timing and are not compared.
-    kStatRxPolls = 3,        // descriptor polling passes of the RX control wavefronts
-    kStatRxNotReady = 4,     // ... of which found no new descriptor
+    // 3..6 are event counts (not stall times) that depend on timing and are not compared.
+    kStatPreparedAhead = 3,  // TX tickets prepared while an earlier payload of the channel was still in flight
+    kStatRxNotReady = 4,     // descriptor polling passes of RX control that found no new descriptor
     kStatTxCreditMiss = 5,   // TX waits for a payload slot ACK or descriptor credit
-    kStatRingFull = 6,       // control waits for a free entry of a ticket ring
+    kStatRingFull = 6,       // control waits for a free entry of a ticket ring (the hand-off stage being busy)
     kStatDescriptors = 7,    // endpoint descriptors published
 };
 

@@ -13,7 +13,8 @@ import torch
 
 from . import _native
 
-FAULT_NONE, FAULT_NO_COUNTS_READY, FAULT_NO_COUNTS_CONSUMED, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE = range(5)
+(FAULT_NONE, FAULT_NO_COUNTS_READY, FAULT_NO_COUNTS_CONSUMED, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE, FAULT_RANK_ORDINAL,
+ FAULT_EXPERT_ORDINAL) = range(7)
 
 
 class PeerGroup:
@@ -32,8 +33,12 @@ class PeerGroup:
             self._runtime.handle, rank, C.c_void_p(x.data_ptr()), C.c_void_p(idx.data_ptr()),
             C.c_void_p(weights.data_ptr()) if weights is not None else None, int(x.shape[0])))
 
-    def start(self, epochs: int = 1, capture: bool = False) -> None:
-        _native.check(self._lib.pcie_ep_peers_start(self._runtime.handle, epochs, 1 if capture else 0), invalid=RuntimeError)
+    def start(self, epochs: int = 1, capture: bool = False, restage: bool = False, read_rows: bool = False) -> None:
+        """Serve the next ``epochs`` dispatches.  ``capture`` keeps what the GPU sent,
+        ``restage`` rewrites every source slot in every epoch (unchanged rows are
+        otherwise left in place), ``read_rows`` makes the receivers read whole rows."""
+        flags = (1 if capture else 0) | (2 if restage else 0) | (4 if read_rows else 0)
+        _native.check(self._lib.pcie_ep_peers_start(self._runtime.handle, epochs, flags), invalid=RuntimeError)
 
     def wait_staged(self, timeout_ms: int = 60_000) -> None:
         _native.check(self._lib.pcie_ep_peers_wait_staged(self._runtime.handle, timeout_ms), invalid=RuntimeError)

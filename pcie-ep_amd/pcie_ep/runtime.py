@@ -85,6 +85,7 @@ class NativeRuntime:
             fuse_receive_expand=int(config.fuse_receive_expand), tx_waves=tx_waves, rx_waves=rx_waves,
             peer_threads=peer_threads, staging_numa_node=staging_numa_node, device=device,
             worker_groups=worker_groups,
+            receive_expand_mode=("pipelined", "vectorized", "scalar").index(config.receive_expand_mode),
         )
         self.native_config = native
         self.sizes = _native.Sizes()

@@ -55,7 +55,7 @@ def test_abi_version_matches_header():
 def test_ctypes_structs_have_the_c_layout(tmp_path):
     """Compile the header as plain C and compare sizeof / offsetof with ctypes."""
     probes = {
-        "pcie_ep_config": (_native.Config, ["num_ranks", "worker_groups", "reserved"]),
+        "pcie_ep_config": (_native.Config, ["num_ranks", "worker_groups", "receive_expand_mode", "reserved", "rank_numa_nodes", "relay_cpus", "relay_delay_ns"]),
         "pcie_ep_sizes": (_native.Sizes, ["unique_rows", "local_experts", "transport_workgroups", "reserved"]),
         "pcie_ep_dispatch_args": (_native.DispatchArgs, ["x", "num_tokens", "plan", "unique_payload", "errors", "prefix_tx_timestamps_ns",
                                                         "expanded_capacity_rows"]),

@@ -21,7 +21,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 @pytest.mark.gpu
 def test_one_json_line_with_roofline_and_cpu_baseline():
-    command = [sys.executable, str(ROOT / "bench.py"), "--tokens", "256", "--steps", "3", "--warmup", "1"]
+    command = [sys.executable, str(ROOT / "bench.py"), "--tokens", "256", "--steps", "3", "--warmup", "1", "--only-headline"]
     print("case: " + " ".join(command[1:]), flush=True)
     outcome = subprocess.run(command, capture_output=True, text=True, timeout=300)
     assert outcome.returncode == 0, outcome.stderr[-2000:]

@@ -4,6 +4,9 @@
 * frozen hotspot top-4 routes of the reference at T=8192 (20 % of the experts
   carry 80 % of the routes) — counts also pinned to the reference's manifest;
 * FP8 wire at T=8192 with heavy-tailed inputs (1 % of the channels x50);
+* the same sizes through the other two output modes: unique rows followed by the
+  stand-alone expand kernel (T=8192 BF16 with alignment 16 and zeroed padding,
+  T=4096 on the FP8 wire) and the unique layout alone (T=8192);
 * cached layout + graph replay sweep, T in {128, 512, 2048, 8192}, 100 replays
   each with fresh payload and weights under fixed routes.
 
@@ -49,6 +52,44 @@ def test_uniform_top8_t4096():
         summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, 8, True, 1, False)
         sent = verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, 8)
         assert summary["expanded"] > 30_000 and sent == summary["stats"][2]
+        del result
+
+
+def test_uniform_top8_t8192_unique_rows_then_expand_kernel():
+    """Receive/expand fusion off: the transport writes unique rows and the
+    stand-alone expand kernel (the reference's scatter_expert_inputs,
+    csrc/kernels/host_staged/dispatch.cuh:8-65) builds the expert-major rows,
+    here with 16-row expert alignment and zeroed gaps."""
+    print("case: uniform top-8 T=8192 bf16, unique rows + expand kernel, alignment 16", flush=True)
+    inputs = baseline_inputs(8192, 8)
+    with make_buffer(8192, 8, fuse_receive_expand=False, receive_expand_mode="scalar") as buffer:
+        result, _ = run_dispatch(buffer, inputs, expand=True, alignment=16, zero_padding=True)
+        summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, 8, True, 16, True)
+        assert summary["expanded"] > 60_000 and summary["unique"] > 40_000
+        assert result[3].receive_expand_overlap is None
+        del result
+
+
+def test_uniform_top8_t8192_unique_layout():
+    """do_expand=False at full size: one row per (source, token) in source order
+    with per-branch local expert ids, -1 elsewhere (layout.cuh:31-48)."""
+    print("case: uniform top-8 T=8192 bf16, unique layout", flush=True)
+    inputs = baseline_inputs(8192, 8)
+    with make_buffer(8192, 8) as buffer:
+        result, _ = run_dispatch(buffer, inputs, expand=False, capture=True)
+        summary = verify_dispatch(result, inputs, 0, WORLD, EXPERTS, 8, False, 1, False)
+        verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, 8)
+        assert summary["unique"] > 40_000
+        del result
+
+
+def test_fp8_wire_t4096_unique_rows_then_expand_kernel():
+    print("case: fp8 wire T=4096 top-8 heavy tail, unique rows + expand kernel", flush=True)
+    inputs = baseline_inputs(4096, 8, heavy_tail=True)
+    with make_buffer(4096, 8, fp8=True, fuse_receive_expand=False, receive_expand_mode="scalar") as buffer:
+        result, _ = run_dispatch(buffer, inputs, expand=True, alignment=8, zero_padding=True, capture=True)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, 8, True, 8, True, fp8_wire=True)
+        verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, 8, fp8_wire=True)
         del result
 
 

@@ -15,7 +15,8 @@ import pytest
 import torch
 
 from helpers import make_inputs, run_dispatch, verify_dispatch
-from pcie_ep.peers import FAULT_NO_COUNTS_CONSUMED, FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE
+from pcie_ep.peers import (FAULT_EXPERT_ORDINAL, FAULT_NO_COUNTS_CONSUMED, FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_RANK_ORDINAL,
+                           FAULT_WRONG_SEQUENCE)
 from test_gpu_dispatch import make_buffer
 
 pytestmark = pytest.mark.gpu
@@ -28,14 +29,14 @@ def small_buffer(**config):
     return make_buffer(tmax=TOKENS, hidden=HIDDEN, channels=2, **config)
 
 
-def failing_dispatch(buffer, inputs, code):
+def failing_dispatch(buffer, inputs, code, expand=True):
     """Dispatch once, expect device error ``code``; the buffer must refuse further work."""
     for source, (x, idx, weights) in enumerate(inputs):
         if source != buffer.rank_idx:
             buffer.peers.set_source(source, x, idx, weights)
     buffer.peers.start(1)
     x, idx, weights = (item.cuda() for item in inputs[buffer.rank_idx])
-    result = buffer.dispatch(x, idx, weights, do_expand=True)
+    result = buffer.dispatch(x, idx, weights, do_expand=expand)
     torch.cuda.synchronize()
     buffer.peers.cancel()
     error = result[3].error.cpu().tolist()
@@ -81,6 +82,18 @@ def test_wrong_payload_identity_is_code_18(inputs):
         buffer.peers.inject_fault(3, FAULT_WRONG_SEQUENCE)
         print("case: rank 3 publishes a descriptor that does not match its slot", flush=True)
         failing_dispatch(buffer, inputs, 18)
+
+
+@pytest.mark.parametrize("fault,expand", [(FAULT_RANK_ORDINAL, False), (FAULT_RANK_ORDINAL, True), (FAULT_EXPERT_ORDINAL, True),
+                                          (FAULT_EXPERT_ORDINAL, False)])
+def test_out_of_range_ordinals_from_a_peer_are_code_18(inputs, fault, expand):
+    """A row whose unique-row or expert ordinal lies outside the counts its source
+    announced would be stored into another expert's rows or before the pool: it is
+    refused like a wrong identity, before any store and without an ACK."""
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(4, fault)
+        print(f"case: rank 4 sends an ordinal beyond its announced counts (fault {fault}, expand={expand})", flush=True)
+        failing_dispatch(buffer, inputs, 18, expand=expand)
 
 
 @pytest.mark.parametrize("which,index", [(0, 0), (1, 1)])
