@@ -156,6 +156,20 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* runtime);
  * submissions the same way: pcie_ep/buffers/ep.py:101, :283). */
 int pcie_ep_dispatch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
 
+/* The same dispatch with the transport scratch (ticket queues, prologue chunk
+ * flags and records, ring history) taken from a fixed array in the library's
+ * device image instead of the runtime's own allocations.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory or do not want
+ * a runtime's scratch allocations in their address map (code under graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  It calls no
+ * allocating routine.  Limits: the scratch a configuration needs (about 0.4 MB at
+ * the defaults; it grows with max_tokens and num_experts) must fit the 4 MiB
+ * array, otherwise PCIE_EP_E_INVALID.  Every runtime on one GPU shares that GPU's
+ * array and each call clears the part that must start at zero, so calls of
+ * different runtimes that overlap in time on one GPU race; per-kernel timing
+ * (pcie_ep_set_kernel_timing) is not recorded by this entry point. */
+int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
+
 /* Thread-local message of the last failing call (runtime may be NULL). */
 const char* pcie_ep_last_error(void);
 

@@ -143,6 +143,14 @@ __global__ void __launch_bounds__(kRowKernelThreads) host_copy_kernel(char* host
     }
 }
 
+// Plain fill: the clearing step of callers that may be under graph capture,
+// where a memset node is not wanted.
+__global__ void __launch_bounds__(kRowKernelThreads) zero_kernel(u32x4* destination, size_t vectors) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors; index += size_t(gridDim.x) * blockDim.x)
+        destination[index] = zero;
+}
+
 int row_grid(int64_t rows, int64_t cap = 8192) {
     // Four wavefronts per workgroup, one row per wavefront, capped so that the
     // grid-stride loop still spreads over all 256 CUs several times.
@@ -160,6 +168,15 @@ hipError_t launch_expand(const DeviceState& state, hipStream_t stream) {
     const dim3 grid(row_grid(unique_capacity(state.z.dims), 16384)), block(kRowKernelThreads);
     if (state.z.dims.hidden % 8 == 0) hipLaunchKernelGGL(expand_kernel<true>, grid, block, 0, stream, state);
     else hipLaunchKernelGGL(expand_kernel<false>, grid, block, 0, stream, state);
+    return hipGetLastError();
+}
+
+hipError_t launch_zero(void* destination, size_t bytes, hipStream_t stream) {
+    if (bytes % 16 || reinterpret_cast<uintptr_t>(destination) % 16) return hipErrorInvalidValue;
+    const size_t vectors = bytes / 16;
+    if (!vectors) return hipSuccess;
+    const size_t blocks = (vectors + kRowKernelThreads - 1) / kRowKernelThreads;
+    hipLaunchKernelGGL(zero_kernel, dim3(unsigned(blocks < 1024 ? blocks : 1024)), dim3(kRowKernelThreads), 0, stream, static_cast<u32x4*>(destination), vectors);
     return hipGetLastError();
 }
 

@@ -42,6 +42,8 @@ int transport_threads(const DeviceState& state);
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
 // Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.
 hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream);
+// Zero `bytes` (a multiple of 16) of device memory at a 16-byte aligned address with a fill kernel.
+hipError_t launch_zero(void* destination, size_t bytes, hipStream_t stream);
 // Kernel-driven copy between pinned host memory and HBM with `wavefronts` wavefronts in flight.
 hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_device, int wavefronts, hipStream_t stream);
 // Stand-alone FP8 wire kernels.

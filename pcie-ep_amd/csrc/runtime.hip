@@ -18,6 +18,7 @@
 #include <cstring>
 #include <fstream>
 #include <memory>
+#include <mutex>
 #include <string>
 
 #include "../../include/pcie_ep_amd.h"
@@ -114,6 +115,52 @@ LaunchShape resolve_launch_shape(const pcie_ep_config& c) {
     return shape;
 }
 
+// ---- static scratch of the allocation-free dispatch --------------------------------
+// One array per GPU, resident from the moment the library's code object is
+// loaded until the process ends.  In host code the array's name is only a
+// stand-in for the symbol: its device address is looked up once per device
+// (static_scratch_of) and every use below goes through that address.
+constexpr size_t kStaticScratchBytes = size_t(4) << 20;
+constexpr int kStaticScratchDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+std::mutex g_scratch_guard;
+unsigned char* g_scratch_address[kStaticScratchDevices] = {};
+
+// Device address of `scratch` on `device`, which must be the current device.
+int static_scratch_of(int device, unsigned char** address) {
+    if (device < 0 || device >= kStaticScratchDevices)
+        return set_error(PCIE_EP_E_INVALID, "device %d is beyond the %d devices the static scratch table covers", device, kStaticScratchDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_guard);
+    if (!g_scratch_address[device]) {
+        void* pointer = nullptr;
+        const hipError_t status = hipGetSymbolAddress(&pointer, HIP_SYMBOL(scratch));
+        if (status != hipSuccess || !pointer)
+            return set_error(PCIE_EP_E_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(status));
+        g_scratch_address[device] = static_cast<unsigned char*>(pointer);
+    }
+    *address = g_scratch_address[device];
+    return 0;
+}
+
+// Carve-out of the transport scratch inside one contiguous block: ticket queues,
+// prologue flags + records, ring history.  Everything from the start of the
+// block up to `clear_bytes` carries epoch-tagged words and must start at zero
+// when the block may have been used by another runtime.
+struct ScratchCarve {
+    size_t queues, layout, history, clear_bytes, bytes;
+};
+ScratchCarve carve_scratch(const SegmentLayout& z) {
+    ScratchCarve c{};
+    c.queues = 0;
+    c.layout = align_up(sizeof(TransportQueues), 256);
+    c.clear_bytes = c.layout + align_up(prologue_flag_bytes(z), 256);
+    c.history = c.layout + align_up(prologue_scratch_bytes(z), 256);
+    const size_t per_channel = size_t(z.dims.max_tokens + z.dims.channels - 1) / z.dims.channels;
+    c.bytes = c.history + align_up(size_t(z.dims.channels) * per_channel * 4, 256);
+    return c;
+}
+
 }  // namespace
 
 struct pcie_ep_runtime {
@@ -130,6 +177,7 @@ struct pcie_ep_runtime {
     int counts_ack_skip_source = -1;
     std::unique_ptr<PeerEmulator> peers;
     uint64_t clock_khz = 100000;  // wall clock of the device, queried at creation
+    unsigned char* static_scratch = nullptr;  // device address of `scratch` on this runtime's GPU
     bool closed = false;
     uint64_t ticks_of_ns(uint64_t ns) const { return ns / 1000000 * clock_khz + ns % 1000000 * clock_khz / 1000000; }
     // Optional per-kernel timing with HIP events on the launch stream.
@@ -298,6 +346,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     HIP_TRY(hipSetDevice(config->device));
     auto rt = std::make_unique<pcie_ep_runtime>();
     rt->config = *config;
+    // Once per device, with that device current: where this GPU keeps its copy of the static scratch.
+    if (int status = static_scratch_of(config->device, &rt->static_scratch)) return status;
     // Every device-side timeout, back-off period and timestamp is derived from the
     // rate of the constant wall clock the kernels read.
     int clock_khz = 0;
@@ -407,6 +457,36 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
         rt->timing_expand = separate_expand;
         rt->timing_valid = true;
     }
+    return 0;
+}
+
+int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, void* stream_handle) {
+    if (!rt) return set_error(PCIE_EP_E_INVALID, "runtime is NULL");
+    DeviceState state;
+    if (int status = build_state(rt, args, state)) return status;
+    const ScratchCarve carve = carve_scratch(rt->z);
+    if (carve.bytes > kStaticScratchBytes)
+        return set_error(PCIE_EP_E_INVALID,
+                         "this configuration needs %zu bytes of transport scratch, more than the %zu bytes of the static scratch; use pcie_ep_dispatch",
+                         carve.bytes, kStaticScratchBytes);
+    // The kernels take the scratch as pointers, exactly as in pcie_ep_dispatch;
+    // here they point into this GPU's static array instead of the runtime's own
+    // allocations.  Only the epoch counter, which is state of the host rings and
+    // not scratch, stays where pcie_ep_runtime_create put it.
+    unsigned char* base = rt->static_scratch;
+    state.queues = reinterpret_cast<TransportQueues*>(base + carve.queues);
+    state.layout_flags = reinterpret_cast<uint64_t*>(base + carve.layout);
+    state.layout_records = reinterpret_cast<int32_t*>(base + carve.layout + prologue_flag_bytes(rt->z));
+    state.chan_remote_tokens = reinterpret_cast<int32_t*>(base + carve.history);
+    hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+    // The array keeps what its last user left, possibly another runtime whose
+    // epoch numbers coincide with this one's: the epoch-tagged words (ticket ring
+    // tags, queue counters, prologue chunk flags) start from zero.  A fill kernel,
+    // not a memset, so the call may be captured into a graph.
+    HIP_TRY(launch_zero(base, carve.clear_bytes, stream));
+    HIP_TRY(launch_prologue(state, stream));
+    HIP_TRY(launch_transport(state, stream));
+    if (state.expand && !state.fuse_expand) HIP_TRY(launch_expand(state, stream));
     return 0;
 }
 

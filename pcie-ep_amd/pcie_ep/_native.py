@@ -59,6 +59,7 @@ _PROTOTYPES = {
     "pcie_ep_runtime_create": (C.c_int, [C.POINTER(Config), C.POINTER(C.c_void_p)]),
     "pcie_ep_runtime_destroy": (C.c_int, [C.c_void_p]),
     "pcie_ep_dispatch": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
+    "pcie_ep_dispatch_static_scratch": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
     "pcie_ep_expand_unique": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
     "pcie_ep_set_test_delays": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64]),
     "pcie_ep_set_test_prefix_delay_ns": (C.c_int, [C.c_void_p, C.c_uint64]),

@@ -96,6 +96,9 @@ class NativeRuntime:
         self.world, self.rank, self.hidden, self.topk = world, rank, hidden, topk
         self.max_tokens, self.experts = max_tokens, experts
         self.channels = config.channels
+        # True routes dispatches through the allocation-free entry point, whose
+        # transport scratch is the library's fixed per-GPU array.
+        self.use_static_scratch = False
         try:
             self._allocate()
             self._lib.pcie_ep_set_test_delays(handle, config.metadata_delay_ns, config.tx_delay_ns, config.rx_delay_ns,
@@ -177,7 +180,8 @@ class NativeRuntime:
         arguments.reuse_plan, arguments.plan = int(cached_layout is not None), plan.storage.data_ptr()
         arguments.expanded_capacity_rows = int(self.sizes.expanded_rows)
         stream = torch.cuda.current_stream(self.device).cuda_stream
-        _native.check(self._lib.pcie_ep_dispatch(self._handle, C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
+        entry = self._lib.pcie_ep_dispatch_static_scratch if self.use_static_scratch else self._lib.pcie_ep_dispatch
+        _native.check(entry(self._handle, C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
         t = pool.tensors
         fused = bool(expand and self.config.fuse_receive_expand)
         result: Dict[str, Any] = {

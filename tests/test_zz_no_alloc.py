@@ -1,0 +1,106 @@
+"""The allocation-free dispatch entry point against the ordinary one.
+
+``pcie_ep_dispatch_static_scratch`` runs the same kernels as ``pcie_ep_dispatch``
+with the transport scratch (ticket queues, prologue flags and records, ring
+history) in the library's fixed per-GPU array.  Every output of the two entry
+points must agree bit for bit on the same inputs, and both with the oracle; the
+static array is reused by consecutive calls (the second with a smaller input, so
+stale contents of the first lie beyond what the second rewrites) and by a second
+runtime whose epoch numbers coincide with the first one's.
+"""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from helpers import make_inputs, run_dispatch, verify_captured, verify_dispatch
+
+pytestmark = pytest.mark.gpu
+
+WORLD, EXPERTS, TOPK, HIDDEN = 8, 64, 4, 1024
+COMPARED = ("unique_count", "expanded_count", "expert_counts", "expert_offsets", "source_offsets", "error")
+
+
+def make_buffer(tmax, **config):
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    config.setdefault("timeout_ms", 5000)
+    return HostStagedEPBuffer(num_max_tokens_per_rank=tmax, hidden=HIDDEN, num_topk=TOPK, num_experts=EXPERTS,
+                              config=HostStagedConfig(channels=4, **config), num_ranks=WORLD, rank=0)
+
+
+def snapshot(result, expand):
+    """Host copies of everything a dispatch defines: the handle's counts and, over
+    the valid row ranges, payload, routes, weights and source metadata."""
+    recv_x, recv_idx, recv_weights, handle, _ = result
+    torch.cuda.synchronize()
+    out = {name: getattr(handle, name).cpu().clone() for name in COMPARED}
+    out["stats"] = handle.stats.cpu()[[0, 1, 2, 7]].clone()
+    if expand:
+        offsets, counts = out["expert_offsets"].tolist(), out["expert_counts"].tolist()
+        rows = torch.cat([torch.arange(offsets[e], offsets[e] + counts[e]) for e in range(len(counts))]) if counts else torch.arange(0)
+    else:
+        rows = torch.arange(int(out["unique_count"]))
+    rows = rows.cuda()
+    out["rows"] = recv_x.view(torch.int16)[rows].cpu()
+    out["idx"] = recv_idx[rows].cpu()
+    out["weights"] = recv_weights[rows].view(torch.int32).cpu()
+    out["meta"] = handle.source_meta[rows].cpu()
+    return out
+
+
+def dispatch_both_ways(buffer, inputs, expand, alignment):
+    """One dispatch through each entry point on the same inputs; returns the two snapshots."""
+    shots = []
+    for static in (False, True):
+        buffer.runtime.use_static_scratch = static
+        print(f"  entry point: {'pcie_ep_dispatch_static_scratch' if static else 'pcie_ep_dispatch'} "
+              f"tokens={[x.shape[0] for x, _, _ in inputs]} expand={expand}", flush=True)
+        result, _ = run_dispatch(buffer, inputs, expand=expand, alignment=alignment, zero_padding=expand, capture=True)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, expand, alignment, expand)
+        verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, TOPK)
+        shots.append(snapshot(result, expand))
+        del result
+    buffer.runtime.use_static_scratch = False
+    return shots
+
+
+def assert_same(ordinary, static):
+    assert ordinary.keys() == static.keys()
+    for name in ordinary:
+        assert torch.equal(ordinary[name], static[name]), f"{name} differs between the two entry points"
+
+
+@pytest.mark.parametrize("expand", [True, False])
+def test_static_scratch_matches_ordinary_dispatch(expand):
+    large = make_inputs(WORLD, [300] * WORLD, HIDDEN, EXPERTS, TOPK, "random", seed=41)
+    small = make_inputs(WORLD, [0] + [37] * (WORLD - 1) if not expand else [53] * WORLD, HIDDEN, EXPERTS, TOPK, "random", seed=42)
+    with make_buffer(300, payload_slots=8, descriptor_slots=4) as buffer:
+        assert_same(*dispatch_both_ways(buffer, large, expand, 8 if expand else 1))
+        # Two static calls in a row, the second smaller than the first.
+        buffer.runtime.use_static_scratch = True
+        for inputs in (large, small):
+            result, _ = run_dispatch(buffer, inputs, expand=expand, alignment=1, zero_padding=expand, capture=True)
+            verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, expand, 1, expand)
+            verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, TOPK)
+            del result
+        buffer.runtime.use_static_scratch = False
+        assert_same(*dispatch_both_ways(buffer, small, expand, 1))
+    # A second runtime starts again at epoch 1 and finds the first one's leftovers
+    # in the shared array.
+    with make_buffer(64) as buffer:
+        assert_same(*dispatch_both_ways(buffer, small if expand else make_inputs(WORLD, [64] * WORLD, HIDDEN, EXPERTS, TOPK, "hotspot", seed=43), expand, 1))
+
+
+def test_static_scratch_rejects_oversized_configuration():
+    """4096 experts with 8192 tokens need more prologue scratch than the array holds."""
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    with HostStagedEPBuffer(num_max_tokens_per_rank=16384, hidden=64, num_topk=2, num_experts=4096,
+                            config=HostStagedConfig(channels=2, timeout_ms=5000, output_pool_size=2), num_ranks=8, rank=0) as buffer:
+        buffer.runtime.use_static_scratch = True
+        x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+        idx = torch.full((4, 2), -1, dtype=torch.int64, device="cuda")
+        with pytest.raises(RuntimeError, match="static scratch"):
+            buffer.dispatch(x, idx, None, do_expand=True)
