@@ -83,7 +83,9 @@ typedef struct pcie_ep_sizes {
     int32_t mailbox_dwords;
     int32_t transport_threads;  /* workgroup size of the transport kernel */
     int32_t transport_workgroups; /* control + payload workgroups; 1..32 more do the local bypass */
-    int32_t reserved[6];
+    int32_t num_domains;        /* NUMA domains of a relay configuration, 0 in direct mode */
+    int32_t reserved[3];
+    int64_t replica_region_bytes; /* one replica payload region (per rank and domain), relay mode */
 } pcie_ep_sizes;
 
 /* One dispatch: inputs, the route plan to fill or reuse, and every output of
@@ -184,12 +186,64 @@ int pcie_ep_set_test_skip_counts_ack_source(pcie_ep_runtime* runtime, int32_t so
  * reference, which has no test of that path. */
 int pcie_ep_set_test_epoch(pcie_ep_runtime* runtime, uint64_t epoch);
 
+/* ---- NUMA relay (numa_mode = 1) ------------------------------------------- */
+
+/* One (channel, domain) flow of this rank's relay workers; the per-flow record
+ * of NumaRelay::diagnostics (csrc/comm/numa_relay.hpp:133-175). */
+typedef struct pcie_ep_relay_flow {
+    int32_t channel;
+    int32_t numa_domain;
+    int32_t worker;             /* index of the worker thread that owns the flow */
+    int32_t cpu;                /* CPU that worker is pinned to, -1 = not pinned */
+    int32_t expected_tokens;    /* rows the flow carries in `epoch` */
+    int32_t error;              /* 0, or 101..106 (also stored in relay_failed) */
+    uint64_t epoch;
+    uint64_t copied_tokens;     /* in `epoch` */
+    uint64_t copied_payload_bytes;
+    uint64_t copy_time_ns_total;
+    uint64_t credit_wait_probes_total;
+    uint64_t drained_epoch;     /* relay_drained[channel][domain] */
+    uint64_t copies_total;      /* since creation */
+    uint64_t payload_bytes_total;
+} pcie_ep_relay_flow;
+
+/* The per-runtime part of AdvancedRuntime::relay_diagnostics (advanced.hpp:182-213). */
+typedef struct pcie_ep_relay_summary {
+    int32_t enabled;
+    int32_t rank;
+    int32_t num_domains;
+    int32_t workers;
+    int32_t flows;              /* flows that exist; at most `capacity` records were written */
+    int32_t source_page_node;   /* node a sampled page of this rank's payload slots resides on, or -errno */
+    int32_t rank_numa_nodes[16];
+    int32_t domain_numa_nodes[8];   /* physical node of every domain */
+    int32_t domain_bound[8];        /* 1: that node exists here and the domain's replica regions were bound to it */
+    int32_t replica_page_node[8];   /* node a sampled page of this rank's replica region of the domain resides on, or -errno */
+    uint64_t epoch;             /* this rank's counts_ready */
+    uint64_t copies;            /* rows copied in `epoch`, all flows */
+    uint64_t payload_bytes;     /* payload bytes copied in `epoch` (metadata and scales excluded) */
+    uint64_t copies_total;
+    uint64_t payload_bytes_total;
+    int64_t slot_stride;
+    int64_t segment_bytes;
+    int64_t replica_region_bytes;
+} pcie_ep_relay_summary;
+
+/* Replaces AdvancedRuntime::relay_diagnostics (advanced.hpp:182-213; csrc/runtime.cu:22).
+ * `flows` may be NULL when capacity is 0.  With numa_mode = 0 only `enabled`,
+ * `rank` and the sizes are filled. */
+int pcie_ep_relay_diagnostics(pcie_ep_runtime* runtime, pcie_ep_relay_summary* summary, pcie_ep_relay_flow* flows, int32_t capacity);
+/* Replaces AdvancedRuntime::set_relay_delay_ns (advanced.hpp:164-167; csrc/runtime.cu:27):
+ * test hook, delays every relay copy of this rank.  PCIE_EP_E_STATE when the relay is not enabled. */
+int pcie_ep_set_relay_delay_ns(pcie_ep_runtime* runtime, uint64_t delay_ns);
+
 /* Replaces get_device_numa_node (advanced_shared_memory.hpp:120-131). */
 int pcie_ep_device_numa_node(int32_t device);
 
 /* Host-visible protocol words, for failure tests that force a condition from
  * the CPU (the reference's destructor does the same store: advanced.hpp:258-261).
- * which: 0 abort, 1 channel_abort[index], 2 counts_ready, 3 counts_consumed[index]. */
+ * which: 0 abort, 1 channel_abort[index], 2 counts_ready, 3 counts_consumed[index],
+ * 4 relay_failed[index], 5 relay_drained[index] (relay mode; index = channel * domains + domain). */
 int pcie_ep_host_signal_store(pcie_ep_runtime* runtime, int32_t segment_rank, int32_t which, int32_t index, uint64_t value);
 int pcie_ep_host_signal_load(pcie_ep_runtime* runtime, int32_t segment_rank, int32_t which, int32_t index, uint64_t* value);
 

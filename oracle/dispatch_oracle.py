@@ -63,16 +63,38 @@ class SourceLayout:
         remote = self.destination_mask & ~np.uint64(1 << own_rank)
         return np.nonzero(remote)[0].astype(np.int32)
 
-    def source_statistics(self, own_rank: int) -> dict:
+    def source_statistics(self, own_rank: int, rank_numa_nodes: Optional[Sequence[int]] = None) -> dict:
         """stats[0], stats[2], stats[7] of the source side
-        (advanced_dispatch.cuh:338, :348-349; tests/test_correctness.py:145-154)."""
+        (advanced_dispatch.cuh:338, :348-349; tests/test_correctness.py:145-154).
+
+        With a NUMA map (relay mode) a token is published once per destination
+        rank of the source's own domain and once per *other* domain it reaches
+        (advanced_common.cuh:207-225), so fewer descriptors than deliveries; the
+        relay workers copy it once per other domain (tests/test_relay.py:16-22)."""
         remote = self.destination_mask & ~np.uint64(1 << own_rank)
         deliveries = int(sum(int(bin(int(m)).count("1")) for m in remote)) if self.tokens else 0
+        descriptors, copies = deliveries, 0
+        if rank_numa_nodes is not None:
+            domains = numa_domains(rank_numa_nodes)
+            descriptors = 0
+            for mask in remote:
+                ranks = [r for r in range(len(domains)) if (int(mask) >> r) & 1]
+                other = {domains[r] for r in ranks} - {domains[own_rank]}
+                descriptors += sum(1 for r in ranks if domains[r] == domains[own_rank]) + len(other)
+                copies += len(other)
         return {
             "host_payload_writes": int(np.count_nonzero(remote)),
             "remote_deliveries": deliveries,
-            "descriptors_published": deliveries,
+            "descriptors_published": descriptors,
+            "relay_copies": copies,
         }
+
+
+def numa_domains(rank_numa_nodes: Sequence[int]) -> list:
+    """Domain index of every rank: the distinct known nodes in ascending order,
+    ranks of unknown node (-1) in domain 0 (advanced_shared_memory.hpp:98-105)."""
+    nodes = sorted({node for node in rank_numa_nodes if node >= 0}) or [0]
+    return [nodes.index(node) if node in nodes else 0 for node in rank_numa_nodes]
 
 
 def source_layout(topk_idx: np.ndarray, num_ranks: int, num_experts: int) -> SourceLayout:
@@ -287,12 +309,13 @@ class DispatchExpectation:
     stats: np.ndarray  # [8] int64; only fields 0, 1, 2 and 7 are deterministic
 
 
-def expected_dispatch(all_idx: Sequence[np.ndarray], rank: int, num_ranks: int, num_experts: int, alignment: int = 1) -> DispatchExpectation:
+def expected_dispatch(all_idx: Sequence[np.ndarray], rank: int, num_ranks: int, num_experts: int, alignment: int = 1,
+                      rank_numa_nodes: Optional[Sequence[int]] = None) -> DispatchExpectation:
     layouts = [source_layout(idx, num_ranks, num_experts) for idx in all_idx]
     receiver = receiver_layout(layouts, rank, num_ranks, num_experts, alignment)
     expanded = expand_rows(layouts, receiver, rank, num_ranks, num_experts)
     unique = unique_rows(layouts, receiver, rank, num_ranks, num_experts)
-    own = layouts[rank].source_statistics(rank)
+    own = layouts[rank].source_statistics(rank, rank_numa_nodes)
     stats = np.zeros(8, dtype=np.int64)
     stats[0] = own["host_payload_writes"]
     stats[1] = receiver.host_payload_reads

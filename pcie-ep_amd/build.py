@@ -24,7 +24,7 @@ CLIENT = OUT_DIR / "abi_client"
 OBJ_DIR = HERE / "build"
 
 HIP_SOURCES = ["prologue_kernel.hip", "transport_kernel.hip", "expand_kernels.hip", "runtime.hip"]
-CXX_SOURCES = ["peers.cpp"]
+CXX_SOURCES = ["peers.cpp", "relay.cpp"]
 
 COMMON = ["-O3", "-std=c++20", "-fPIC", "-Wall", "-Wno-unused-function", "-pthread"]
 # Packed FP32 instructions are disabled for all device code of this build.

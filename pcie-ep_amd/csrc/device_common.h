@@ -34,16 +34,16 @@ struct alignas(16) RxEntry {
     int32_t channel;
     uint64_t payload_sequence;
     int32_t channel_ordinal;  // position among the channel's receive tickets of this dispatch
-    int32_t reserved;
+    int32_t replica;          // 1: `slot` is a replica slot of this rank's domain (relay mode)
 };
 struct alignas(16) TxEntry {
     int32_t token;
     int32_t ordinal;  // position among this channel's remote tokens
-    uint32_t endpoints;
+    uint32_t endpoints;  // destination ranks of the own domain and, in relay mode, relay endpoints P + domain
     int32_t channel;
-    int32_t descriptor_ordinal[kMaxRanks];
+    int32_t descriptor_ordinal[kMaxEndpoints];
 };
-static_assert(sizeof(RxEntry) == 32 && sizeof(TxEntry) == 80, "queue entry layout");
+static_assert(sizeof(RxEntry) == 32 && sizeof(TxEntry) == 112, "queue entry layout");
 
 struct alignas(128) QueueCounter {
     uint32_t value;
@@ -70,6 +70,7 @@ struct alignas(256) TransportQueues {
 struct DeviceState {
     SegmentLayout z;
     char* seg[kMaxRanks];
+    char* replica_in[kMaxRanks];  // relay mode: replica payload region of every source for this rank's domain
     int local_rank;
     int fuse_expand;  // receive waves scatter straight into expert rows
     int expand;
@@ -95,6 +96,7 @@ struct DeviceState {
     int32_t* plan_counts;     // [P + E]
     int32_t* plan_chan_counts;// [C, P]
     int32_t* plan_chan_remote;// [C]
+    int32_t* plan_chan_relay; // [C, N]: own tokens of each channel bound for each other domain (relay mode)
 
     int32_t* chan_remote_tokens;  // scratch [C, ceil(Tmax / C)]: ring history for slot reuse
     TransportQueues* queues;
@@ -307,20 +309,23 @@ __device__ __forceinline__ uint64_t lanes_below(int lane) { return lane >= 64 ? 
 __device__ __forceinline__ int broadcast_first(int value) { return __builtin_amdgcn_readfirstlane(value); }
 
 // ---- abort flags on the host segments ----------------------------------------------
-// Flags per rank: abort, then channel_abort[C].  All 64 lanes load in parallel
-// (the reference scans 32 at a time: advanced_common.cuh:350-378).  A scan may be
-// restricted to the flags whose index is congruent to `slice` modulo `slices`.
+// Flags per rank: abort, channel_abort[C] and, in relay mode, relay_failed[C][N].
+// All 64 lanes load in parallel (the reference scans 32 at a time:
+// advanced_common.cuh:350-378).  A scan may be restricted to the flags whose
+// index is congruent to `slice` modulo `slices`.
+__device__ __forceinline__ int abort_flags_per_rank(const SegmentLayout& z) { return 1 + z.dims.channels * (1 + z.dims.domains); }
+__device__ __forceinline__ const uint64_t* abort_flag_at(const SegmentLayout& z, char* segment, int flag) {
+    if (flag == 0) return signal_at(segment, z.abort_offset);
+    if (flag <= z.dims.channels) return signal_at(segment, z.channel_abort_offset, flag - 1);
+    return signal_at(segment, z.relay_failed_offset, flag - 1 - z.dims.channels);
+}
 __device__ inline bool any_abort_wave(const DeviceState& state, int lane, int slice = 0, int slices = 1) {
-    const int per_rank = 1 + state.z.dims.channels;
+    const int per_rank = abort_flags_per_rank(state.z);
     const int flags = state.z.dims.num_ranks * per_rank;
     bool aborted = false;
     for (int index = lane; index < flags; index += kWave) {
         if (index % slices != slice) continue;
-        char* segment = state.seg[index / per_rank];
-        const int flag = index % per_rank;
-        const uint64_t* signal = flag == 0 ? signal_at(segment, state.z.abort_offset)
-                                           : signal_at(segment, state.z.channel_abort_offset, flag - 1);
-        aborted |= host_load(signal) != 0;
+        aborted |= host_load(abort_flag_at(state.z, state.seg[index / per_rank], index % per_rank)) != 0;
     }
     return __any(aborted);
 }

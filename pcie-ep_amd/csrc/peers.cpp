@@ -76,9 +76,22 @@ void host_dequantize_fp8(const uint8_t* codes, const float* scales, uint16_t* ou
             out[size_t(token) * hidden + i] = fp8_dequantize_element(codes[size_t(token) * hidden + i], scales[token]);
 }
 
-PeerEmulator::PeerEmulator(const SegmentLayout& layout, int local_rank, char* const* segments, int threads, int timeout_ms)
+PeerEmulator::PeerEmulator(const SegmentLayout& layout, int local_rank, char* const* segments, char* const* replica, int threads,
+                           int timeout_ms, const RelayOptions& relay)
     : z_(layout), me_(local_rank), timeout_ms_(timeout_ms), ranks_(layout.dims.num_ranks) {
     for (int rank = 0; rank < kMaxRanks; ++rank) seg_[rank] = rank < z_.dims.num_ranks ? segments[rank] : nullptr;
+    for (int rank = 0; rank < z_.dims.num_ranks; ++rank)
+        for (int domain = 0; domain < z_.dims.domains; ++domain) replica_[rank][domain] = replica[rank * kMaxDomains + domain];
+    if (z_.dims.domains) {
+        // The relay workers an emulated source's own process would run.  Only the
+        // GPU consumes what they publish: the other receivers are not simulated.
+        RelayOptions options = relay;
+        options.live_ranks = 1u << me_;
+        options.workers_per_domain = 1;
+        options.pin = false;
+        for (int rank = 0; rank < z_.dims.num_ranks; ++rank)
+            if (rank != me_) relays_.push_back(std::make_unique<NumaRelay>(z_, rank, seg_, replica_[rank], options));
+    }
     const int channels = z_.dims.channels;
     for (auto& state : ranks_) {
         state.remote.resize(channels);
@@ -105,6 +118,7 @@ PeerEmulator::PeerEmulator(const SegmentLayout& layout, int local_rank, char* co
 }
 
 PeerEmulator::~PeerEmulator() {
+    for (auto& relay : relays_) relay->stop_and_join();
     {
         std::lock_guard<std::mutex> lock(mutex_);
         stop_ = true;
@@ -202,7 +216,9 @@ int PeerEmulator::wait_staged(int timeout_ms, std::string& error) {
 
 int PeerEmulator::wait(int timeout_ms, std::string& error) {
     std::unique_lock<std::mutex> lock(mutex_);
-    const bool finished = finished_.wait_for(lock, std::chrono::milliseconds(timeout_ms), [this] {
+    // A deadline on the system clock: this form of the wait goes through
+    // pthread_cond_timedwait, which thread-checking tools understand.
+    const bool finished = finished_.wait_until(lock, std::chrono::system_clock::now() + std::chrono::milliseconds(timeout_ms), [this] {
         for (uint64_t done : thread_done_) if (done != target_) return false;
         return true;
     });
@@ -336,7 +352,7 @@ void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int chan
             state.slot_token[slot_index] = -1;  // stage the true row again next time
         }
     }
-    Descriptor* descriptor = descriptor_at(z_, own, channel, me_, ordinal);
+    Descriptor* descriptor = descriptor_at(z_, own, channel, endpoint_of(z_.dims, rank, me_), ordinal);
     descriptor->payload_slot = slot;
     // The token identifies the payload (its sequence is sequence(epoch, token));
     // the fault hook publishes a token that does not match the slot's metadata.
@@ -361,6 +377,15 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
         // The GPU must have consumed the previous mailbox before it is rewritten
         // (advanced_layout.cuh:60-88 from the source's point of view).
         if (epoch > 1 && acquire(signal_at(own, z_.counts_consumed_offset, me_)) != epoch - 1) { quiescent = true; return false; }
+        // ... and so must this source's relay flows have (advanced_dispatch.cuh:213-225).
+        if (epoch > 1 && !relays_drained(rank, epoch - 1)) { quiescent = true; return false; }
+        // Relay mode: rows for the GPU travel through the relay endpoint of the
+        // GPU's domain when this source sits in another one.
+        for (int domain = 0; domain < z_.dims.domains; ++domain) {
+            const bool carries = reads_replica(z_.dims, rank, me_) && domain == z_.dims.rank_domain[me_];
+            for (int channel = 0; channel < channels; ++channel)
+                relay_mailbox_at(z_, own, domain)[channel] = carries ? state.channel_counts[size_t(channel) * ranks + me_] : 0;
+        }
         for (int destination = 0; destination < ranks; ++destination) {
             int32_t* block = mailbox_at(z_, own, destination);
             block[0] = state.counts[destination];
@@ -372,6 +397,7 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
         state.source_phase = 1;
         progressed = true;
     }
+    const int endpoint = endpoint_of(z_.dims, rank, me_);
     if (state.source_phase == 1) {
         bool all_published = true;
         for (int channel = 0; channel < channels; ++channel) {
@@ -387,11 +413,11 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
                     // occupant is not necessarily the one whose ACK matters.
                     const size_t slot_index = size_t(channel) * slots + slot;
                     if (state.pending_sequence[slot_index]) {
-                        if (acquire(ack_at(z_, own, channel, slot, me_)) != state.pending_sequence[slot_index]) break;
+                        if (acquire(ack_at(z_, own, channel, slot, endpoint)) != state.pending_sequence[slot_index]) break;
                         state.pending_sequence[slot_index] = 0;
                     }
                     const int ordinal = state.sent[channel];
-                    if (!credit_covers(acquire(credit_at(z_, own, channel, me_)), epoch, ordinal, descriptors)) break;
+                    if (!credit_covers(acquire(credit_at(z_, own, channel, endpoint)), epoch, ordinal, descriptors)) break;
                     // Row faults apply to the last row this source sends to the GPU on the channel.
                     const bool last = state.sent[channel] + 1 == state.channel_counts[size_t(channel) * ranks + me_];
                     publish_token(state, rank, epoch, channel, token, slot, ordinal, last ? fault : kFaultNone);
@@ -414,7 +440,7 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
         size_t kept = 0;
         for (int slot_index : state.pending_slots) {
             const uint64_t expected = state.pending_sequence[slot_index];
-            if (expected && acquire(signal_at(own, z_.ack_offset, size_t(slot_index) * ranks + me_)) != expected) {
+            if (expected && acquire(signal_at(own, z_.ack_offset, size_t(slot_index) * z_.endpoints + endpoint)) != expected) {
                 state.pending_slots[kept++] = slot_index;
             } else {
                 state.pending_sequence[slot_index] = 0;
@@ -423,7 +449,8 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
             }
         }
         state.pending_slots.resize(kept);
-        if (state.pending_slots.empty()) {
+        // The epoch is over for this source once its relay flows are drained too.
+        if (state.pending_slots.empty() && relays_drained(rank, epoch)) {
             state.source_phase = 3;
             done = true;
         }
@@ -439,6 +466,8 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
     char* gpu = seg_[me_];
     const int channels = z_.dims.channels, local = z_.local_experts, topk = z_.dims.topk;
     const int fault = state.fault.load(std::memory_order_relaxed);
+    const bool replica = reads_replica(z_.dims, me_, rank);
+    const int domain = z_.dims.domains ? z_.dims.rank_domain[rank] : 0;
     bool progressed = false;
     if (state.receiver_phase == 0) {
         if (acquire(signal_at(gpu, z_.counts_ready_offset)) != epoch) return false;
@@ -462,15 +491,18 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
         for (int channel = 0; channel < channels; ++channel) {
             while (state.consumed[channel] < state.expected[channel]) {
                 const int ordinal = state.consumed[channel];
-                Descriptor* descriptor = descriptor_at(z_, gpu, channel, rank, ordinal);
+                // A receiver of another domain than the GPU's reads the replica ring
+                // that the GPU's relay workers fill for its domain.
+                Descriptor* descriptor = replica ? replica_descriptor_at(z_, gpu, channel, domain, rank, ordinal)
+                                                 : descriptor_at(z_, gpu, channel, rank, ordinal);
                 if (acquire(&descriptor->ready) != sequence(epoch, ordinal)) break;
                 const int slot = descriptor->payload_slot, token = descriptor->token_index;
                 const uint64_t payload_sequence = sequence(epoch, token);
-                if (slot < 0 || slot >= z_.dims.payload_slots || token < 0 || token >= z_.dims.max_tokens) {
+                if (slot < 0 || slot >= (replica ? z_.dims.replica_slots : z_.dims.payload_slots) || token < 0 || token >= z_.dims.max_tokens) {
                     error = "GPU published a descriptor with an out-of-range slot or token";
                     return false;
                 }
-                const char* base = slot_at(z_, gpu, channel, slot);
+                const char* base = replica ? replica_slot_at(z_, replica_[me_][domain], channel, slot) : slot_at(z_, gpu, channel, slot);
                 SlotMetaHeader header;
                 std::memcpy(&header, base + z_.meta_offset, sizeof header);
                 if (header.token_index != token) {
@@ -504,8 +536,9 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
                 }
                 std::atomic_thread_fence(std::memory_order_seq_cst);
                 const bool last = state.receive_done + 1 == state.receive_total;
-                if (!(fault == kFaultWithholdLastAck && last)) release(ack_at(z_, gpu, channel, slot, rank), payload_sequence);
-                release(credit_at(z_, gpu, channel, rank), sequence(epoch, ordinal));
+                if (!(fault == kFaultWithholdLastAck && last))
+                    release(replica ? replica_ack_at(z_, gpu, channel, domain, slot, rank) : ack_at(z_, gpu, channel, slot, rank), payload_sequence);
+                release(replica ? replica_credit_at(z_, gpu, channel, domain, rank) : credit_at(z_, gpu, channel, rank), sequence(epoch, ordinal));
                 ++state.consumed[channel];
                 ++state.receive_done;
                 progressed = true;
@@ -518,6 +551,13 @@ bool PeerEmulator::receiver_progress(int rank, uint64_t epoch, bool& done, std::
     }
     if (state.receiver_phase == 2) done = true;
     return progressed;
+}
+
+bool PeerEmulator::relays_drained(int rank, uint64_t epoch) const {
+    for (int channel = 0; channel < z_.dims.channels; ++channel)
+        for (int domain = 0; domain < z_.dims.domains; ++domain)
+            if (acquire(signal_at(seg_[rank], z_.relay_drained_offset, flow_index(z_, channel, domain))) != epoch) return false;
+    return true;
 }
 
 int64_t PeerEmulator::captured_count(int rank) {

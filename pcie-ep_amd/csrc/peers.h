@@ -18,6 +18,7 @@
 #include <thread>
 #include <vector>
 
+#include "relay.h"
 #include "wire.h"
 
 namespace pcie_ep {
@@ -47,7 +48,11 @@ enum PeerFlag : uint32_t {
 
 class PeerEmulator {
 public:
-    PeerEmulator(const SegmentLayout& layout, int local_rank, char* const* segments, int threads, int timeout_ms);
+    // `replica[rank * kMaxDomains + domain]` is the replica payload region of
+    // `rank` for `domain` (relay mode; unused otherwise).  In relay mode every
+    // emulated source gets relay workers of its own, as its process would have.
+    PeerEmulator(const SegmentLayout& layout, int local_rank, char* const* segments, char* const* replica, int threads, int timeout_ms,
+                 const RelayOptions& relay);
     ~PeerEmulator();
 
     int set_source(int rank, const uint16_t* x, const int64_t* topk_idx, const float* weights, int tokens, std::string& error);
@@ -102,9 +107,13 @@ private:
     void publish_token(Rank& state, int rank, uint64_t epoch, int channel, int token, int slot, int ordinal, int fault);
     void fail(const std::string& message);
 
+    bool relays_drained(int rank, uint64_t epoch) const;
+
     SegmentLayout z_;
     int me_;
     char* seg_[kMaxRanks];
+    char* replica_[kMaxRanks][kMaxDomains] = {};
+    std::vector<std::unique_ptr<NumaRelay>> relays_;  // one per emulated source (relay mode)
     int timeout_ms_;
     std::vector<Rank> ranks_;
     std::vector<std::thread> threads_;

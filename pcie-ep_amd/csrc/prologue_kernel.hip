@@ -42,6 +42,12 @@ __device__ void publish_counts(const DeviceState& state, uint64_t epoch) {
         else value = state.plan_chan_counts[(field - 1 - local) * ranks + destination];
         host_field_store(mailbox_at(z, own, destination) + field, value);
     }
+    // Relay mode: what each (channel, domain) relay flow of this source will carry.
+    const int domains = z.dims.domains, channels = z.dims.channels;
+    for (int index = threadIdx.x; index < domains * channels; index += blockDim.x) {
+        const int domain = index / channels, channel = index % channels;
+        host_field_store(relay_mailbox_at(z, own, domain) + channel, state.plan_chan_relay[channel * domains + domain]);
+    }
     // Every writer waits for its own stores; the leader publishes after the join
     // (a leader-only wait would not cover the other writers: layout.cuh:21-28).
     wait_memory_ops();
@@ -53,12 +59,13 @@ __device__ void publish_counts(const DeviceState& state, uint64_t epoch) {
 
 // Per-chunk record in the layout scratch (int32 units).
 struct ChunkRecord {
-    int bins, channels, ranks;
-    __host__ __device__ int stride() const { return bins + channels * ranks + channels + 4; }
+    int bins, channels, ranks, domains;
+    __host__ __device__ int stride() const { return error_key() + 4; }
     __host__ __device__ int counts() const { return 0; }
     __host__ __device__ int chan_counts() const { return bins; }
     __host__ __device__ int chan_remote() const { return bins + channels * ranks; }
-    __host__ __device__ int error_key() const { return bins + channels * ranks + channels; }
+    __host__ __device__ int chan_relay() const { return chan_remote() + channels; }
+    __host__ __device__ int error_key() const { return chan_relay() + channels * domains; }
 };
 
 template <int kTopk>
@@ -72,7 +79,8 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     const int chunk = blockIdx.x;
     const bool leader = chunk == 0;
     char* own = state.seg[state.local_rank];
-    const ChunkRecord record{bins, channels, ranks};
+    const int domains = z.dims.domains;
+    const ChunkRecord record{bins, channels, ranks, domains};
     uint64_t* chunk_flags = state.layout_flags;
     int32_t* chunk_records = state.layout_records;
     // The leader bumps the epoch only after every chunk's flag carries this tag,
@@ -112,13 +120,9 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         // Abort signals are terminal, and the previous count mailbox must have
         // been consumed.  Issue the host loads now; the verdicts are taken after
         // the layout so their PCIe latency hides behind it.
-        const int per_rank = 1 + channels;
-        for (int index = threadIdx.x; index < ranks * per_rank; index += blockDim.x) {
-            char* segment = state.seg[index / per_rank];
-            const int flag = index % per_rank;
-            const uint64_t* signal = flag == 0 ? signal_at(segment, z.abort_offset) : signal_at(segment, z.channel_abort_offset, flag - 1);
-            aborted |= host_load(signal) != 0;
-        }
+        const int per_rank = abort_flags_per_rank(z);
+        for (int index = threadIdx.x; index < ranks * per_rank; index += blockDim.x)
+            aborted |= host_load(abort_flag_at(z, state.seg[index / per_rank], index % per_rank)) != 0;
         if (wave == 0 && tag > 1 && lane < ranks && lane != state.local_rank)
             consumed = host_load(signal_at(own, z.counts_consumed_offset, lane)) == tag - 1;
     }
@@ -128,13 +132,15 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     int* base = reinterpret_cast<int*>(masks + size_t(bins) * chunk_waves);    // [bins]
     int* chan_counts = base + bins;                                            // [C][P]
     int* chan_remote = chan_counts + channels * ranks;                         // [C]
-    int* first_error = chan_remote + channels;                                 // lowest token * 64 + branch
+    int* chan_relay = chan_remote + channels;                                  // [C][N]
+    int* first_error = chan_relay + channels * domains;                        // lowest token * 64 + branch
     // Exclusive prefixes inside the chunk never exceed its 1024 tokens: 16 bits each.
     uint16_t* prefix = reinterpret_cast<uint16_t*>(first_error + 2);           // [W][bins]
     if (!state.reuse_plan && chunk < chunks) {
         for (int i = threadIdx.x; i < bins * chunk_waves; i += blockDim.x) masks[i] = 0;
         for (int i = threadIdx.x; i < channels * ranks; i += blockDim.x) chan_counts[i] = 0;
         for (int i = threadIdx.x; i < channels; i += blockDim.x) chan_remote[i] = 0;
+        for (int i = threadIdx.x; i < channels * domains; i += blockDim.x) chan_relay[i] = 0;
         if (threadIdx.x == 0) *first_error = 0x7FFFFFFF;
         __syncthreads();
         const int tokens = state.num_tokens;
@@ -176,6 +182,11 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
             for (int rank = 0; rank < ranks; ++rank)
                 if ((destination_mask >> rank) & 1u) atomicAdd(chan_counts + channel * ranks + rank, 1);
             if (destination_mask & ~(1u << state.local_rank)) atomicAdd(chan_remote + channel, 1);
+            // Relay endpoints of the token: one per other domain it reaches
+            // (the endpoint counts of advanced_layout.cuh:405-412).
+            const uint32_t relayed = endpoint_mask_of(z.dims, state.local_rank, destination_mask) >> ranks;
+            for (int domain = 0; domain < domains; ++domain)
+                if ((relayed >> domain) & 1u) atomicAdd(chan_relay + channel * domains + domain, 1);
         }
         __syncthreads();
         // Publish this chunk's totals, then its flag.
@@ -190,6 +201,7 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         }
         for (int i = threadIdx.x; i < channels * ranks; i += blockDim.x) device_store(mine + record.chan_counts() + i, chan_counts[i]);
         for (int i = threadIdx.x; i < channels; i += blockDim.x) device_store(mine + record.chan_remote() + i, chan_remote[i]);
+        for (int i = threadIdx.x; i < channels * domains; i += blockDim.x) device_store(mine + record.chan_relay() + i, chan_relay[i]);
         if (threadIdx.x == 0) device_store(mine + record.error_key(), *first_error);
         wait_memory_ops();
         __syncthreads();
@@ -252,13 +264,14 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         }
         __syncthreads();
         if (!stalled) {
-            const int fields = record.error_key();  // counts, channel counts, channel remote tokens
+            const int fields = record.error_key();  // counts, channel counts, channel remote tokens, relay counts
             for (int field = threadIdx.x; field < fields; field += blockDim.x) {
                 int sum = 0;
                 for (int other = 0; other < chunks; ++other) sum += device_load(chunk_records + size_t(other) * record.stride() + field);
                 if (field < bins) state.plan_counts[field] = sum;
                 else if (field < record.chan_remote()) state.plan_chan_counts[field - record.chan_counts()] = sum;
-                else state.plan_chan_remote[field - record.chan_remote()] = sum;
+                else if (field < record.chan_relay()) state.plan_chan_remote[field - record.chan_remote()] = sum;
+                else state.plan_chan_relay[field - record.chan_relay()] = sum;
             }
             if (threadIdx.x == 0) {
                 int key = 0x7FFFFFFF;
@@ -320,7 +333,8 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
 
 size_t prologue_lds_bytes(const SegmentLayout& z, int chunk_waves) {
     const size_t bins = size_t(z.dims.num_ranks) + z.dims.num_experts;
-    return bins * chunk_waves * 10 + bins * 4 + size_t(z.dims.channels) * z.dims.num_ranks * 4 + size_t(z.dims.channels) * 4 + 64;
+    return bins * chunk_waves * 10 + bins * 4 + size_t(z.dims.channels) * z.dims.num_ranks * 4 +
+           size_t(z.dims.channels) * (1 + z.dims.domains) * 4 + 64;
 }
 
 // The largest chunk whose tables fit the 64 KiB of LDS every workgroup may use
@@ -340,7 +354,7 @@ int prologue_chunks(const SegmentLayout& z, int tokens) {
 size_t prologue_flag_bytes(const SegmentLayout& z) { return align_up(size_t(prologue_chunks(z, z.dims.max_tokens)) * 8, 256); }
 
 size_t prologue_scratch_bytes(const SegmentLayout& z) {
-    const ChunkRecord record{z.dims.num_ranks + z.dims.num_experts, z.dims.channels, z.dims.num_ranks};
+    const ChunkRecord record{z.dims.num_ranks + z.dims.num_experts, z.dims.channels, z.dims.num_ranks, z.dims.domains};
     return prologue_flag_bytes(z) + size_t(prologue_chunks(z, z.dims.max_tokens)) * record.stride() * 4;
 }
 

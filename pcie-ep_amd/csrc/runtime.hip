@@ -13,10 +13,13 @@
 #include <unistd.h>
 
 #include <cctype>
+#include <cerrno>
+#include <vector>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
+#include <algorithm>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -24,6 +27,7 @@
 #include "../../include/pcie_ep_amd.h"
 #include "launch.h"
 #include "peers.h"
+#include "relay.h"
 
 using namespace pcie_ep;
 
@@ -50,7 +54,7 @@ int set_error(int code, const char* format, ...) {
 
 // Plan blob sub-layout (the tensors of AdvancedLayout: advanced.hpp:21-41).
 struct PlanLayout {
-    size_t mask, rank_ord, exp_idx, exp_ord, counts, chan_counts, chan_remote, bytes;
+    size_t mask, rank_ord, exp_idx, exp_ord, counts, chan_counts, chan_remote, chan_relay, bytes;
 };
 
 PlanLayout plan_layout(const Dimensions& d) {
@@ -69,8 +73,27 @@ PlanLayout plan_layout(const Dimensions& d) {
     p.counts = reserve(size_t(d.num_ranks + d.num_experts) * 4);
     p.chan_counts = reserve(size_t(d.channels) * d.num_ranks * 4);
     p.chan_remote = reserve(size_t(d.channels) * 4);
+    p.chan_relay = reserve(size_t(d.channels) * (d.domains ? d.domains : 1) * 4);
     p.bytes = cursor;
     return p;
+}
+
+// Domains of a relay configuration: the distinct known nodes of the ranks in
+// ascending order (one placeholder domain when none is known); a rank of unknown
+// node belongs to domain 0 (advanced_shared_memory.hpp:98-105).
+int numa_domains(const pcie_ep_config& c, int* nodes, int* rank_domain) {
+    int count = 0;
+    for (int rank = 0; rank < c.num_ranks; ++rank) {
+        const int node = c.rank_numa_nodes[rank];
+        if (node >= 0 && std::find(nodes, nodes + count, node) == nodes + count) nodes[count++] = node;
+    }
+    if (!count) nodes[count++] = 0;
+    std::sort(nodes, nodes + count);
+    for (int rank = 0; rank < c.num_ranks; ++rank) {
+        const int* found = std::find(nodes, nodes + count, c.rank_numa_nodes[rank]);
+        rank_domain[rank] = found == nodes + count ? 0 : int(found - nodes);
+    }
+    return count;
 }
 
 int check_config(const pcie_ep_config* c, Dimensions& dims) {
@@ -95,6 +118,18 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
     if (c->staging_numa_node < -1 || c->staging_numa_node >= 1024) return set_error(PCIE_EP_E_INVALID, "staging_numa_node must be -1..1023");
     dims = Dimensions{c->num_ranks, c->max_tokens, c->hidden, c->topk, c->num_experts, c->channels, c->payload_slots, c->descriptor_slots,
                       c->wire_fp8 ? 1 : 0};
+    if (c->numa_mode != 0 && c->numa_mode != 1) return set_error(PCIE_EP_E_INVALID, "invalid NUMA mode");
+    if (c->numa_mode == 1) {
+        // advanced_shared_memory.hpp:96-111
+        if (c->replica_slots <= 0) return set_error(PCIE_EP_E_INVALID, "invalid advanced capacity or timeout");
+        if (c->relay_workers_per_numa < 1 || c->relay_workers_per_numa > c->channels) return set_error(PCIE_EP_E_INVALID, "invalid relay worker count");
+        if (c->relay_cpu_count < 0 || c->relay_cpu_count > 64) return set_error(PCIE_EP_E_INVALID, "relay_cpu_count must be 0..64");
+        int nodes[kMaxRanks];
+        const int count = numa_domains(*c, nodes, dims.rank_domain);
+        if (count > kMaxDomains) return set_error(PCIE_EP_E_INVALID, "too many NUMA domains");
+        dims.domains = count;
+        dims.replica_slots = c->replica_slots;
+    }
     return 0;
 }
 
@@ -161,6 +196,27 @@ ScratchCarve carve_scratch(const SegmentLayout& z) {
     return c;
 }
 
+// One pinned, fine-grained, GPU-mapped allocation, first touched (and zeroed)
+// under a bind policy for `node` when node >= 0.
+int pinned_zeroed(size_t bytes, int node, char** out, const char* what) {
+    unsigned long node_mask[16] = {};
+    const bool bind = node >= 0;
+    if (bind) {
+        if (node >= 1024) return set_error(PCIE_EP_E_INVALID, "NUMA node %d is out of range", node);
+        node_mask[node / 64] = 1ul << (node % 64);
+        if (syscall(SYS_set_mempolicy, MPOL_BIND, node_mask, sizeof(node_mask) * 8) != 0)
+            return set_error(PCIE_EP_E_INVALID, "set_mempolicy(MPOL_BIND, node %d) failed", node);
+    }
+    void* pointer = nullptr;
+    const unsigned flags = hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable | (bind ? hipHostMallocNumaUser : 0u);
+    const hipError_t allocated = hipHostMalloc(&pointer, bytes, flags);
+    if (allocated == hipSuccess) std::memset(pointer, 0, bytes);
+    if (bind) syscall(SYS_set_mempolicy, MPOL_DEFAULT, nullptr, 0);
+    if (allocated != hipSuccess) return set_error(PCIE_EP_E_HIP, "hipHostMalloc of a %zu-byte %s failed: %s", bytes, what, hipGetErrorString(allocated));
+    *out = static_cast<char*>(pointer);
+    return 0;
+}
+
 }  // namespace
 
 struct pcie_ep_runtime {
@@ -175,6 +231,12 @@ struct pcie_ep_runtime {
     char* layout_scratch = nullptr;
     uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
     int counts_ack_skip_source = -1;
+    // Relay mode: replica payload regions [rank][domain], each bound to its
+    // domain's node when that node exists here, and this rank's relay workers.
+    char* replica[kMaxRanks * kMaxDomains] = {};
+    int domain_node[kMaxDomains] = {};
+    bool domain_bound[kMaxDomains] = {};
+    std::unique_ptr<NumaRelay> relay;
     std::unique_ptr<PeerEmulator> peers;
     uint64_t clock_khz = 100000;  // wall clock of the device, queried at creation
     unsigned char* static_scratch = nullptr;  // device address of `scratch` on this runtime's GPU
@@ -229,7 +291,10 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
 
     std::memset(&s, 0, sizeof s);
     s.z = rt->z;
-    for (int rank = 0; rank < d.num_ranks; ++rank) s.seg[rank] = rt->segments[rank];
+    for (int rank = 0; rank < d.num_ranks; ++rank) {
+        s.seg[rank] = rt->segments[rank];
+        if (d.domains) s.replica_in[rank] = rt->replica[rank * kMaxDomains + d.rank_domain[rt->config.local_rank]];
+    }
     s.local_rank = rt->config.local_rank;
     s.queues = rt->queues;
     s.worker_groups = rt->worker_groups;
@@ -264,6 +329,7 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.plan_counts = reinterpret_cast<int32_t*>(plan + rt->plan.counts);
     s.plan_chan_counts = reinterpret_cast<int32_t*>(plan + rt->plan.chan_counts);
     s.plan_chan_remote = reinterpret_cast<int32_t*>(plan + rt->plan.chan_remote);
+    s.plan_chan_relay = reinterpret_cast<int32_t*>(plan + rt->plan.chan_relay);
     s.chan_remote_tokens = rt->chan_remote_tokens;
     s.layout_flags = reinterpret_cast<uint64_t*>(rt->layout_scratch);
     s.layout_records = reinterpret_cast<int32_t*>(rt->layout_scratch + prologue_flag_bytes(rt->z));
@@ -332,6 +398,8 @@ int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes) {
     probe.worker_groups = shape.worker_groups;
     sizes->transport_threads = transport_threads(probe);
     sizes->transport_workgroups = config->channels + probe.worker_groups;
+    sizes->num_domains = dims.domains;
+    sizes->replica_region_bytes = dims.domains ? int64_t(z.replica_region_bytes) : 0;
     return 0;
 }
 
@@ -364,27 +432,26 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers
     // /dev/shm mappings: advanced_shared_memory.hpp:264-288).  First touch is
     // by this thread under the requested NUMA policy, then zeroed: a zero
-    // sequence word means "never written".
-    const bool bind = config->staging_numa_node >= 0;
-    unsigned long node_mask[16] = {};
-    if (bind) {
-        node_mask[config->staging_numa_node / 64] = 1ul << (config->staging_numa_node % 64);
-        if (syscall(SYS_set_mempolicy, MPOL_BIND, node_mask, sizeof(node_mask) * 8) != 0)
-            return set_error(PCIE_EP_E_INVALID, "set_mempolicy(MPOL_BIND, node %d) failed", config->staging_numa_node);
-    }
+    // sequence word means "never written".  In relay mode a rank's segment
+    // belongs on the rank's own node and each replica payload region on the node
+    // of the domain it serves (advanced_shared_memory.hpp:214-262); a node that
+    // this machine does not have leaves the memory where first touch puts it.
     int status = 0;
-    for (int rank = 0; rank < dims.num_ranks && !status; ++rank) {
-        void* pointer = nullptr;
-        const unsigned flags = hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable | (bind ? hipHostMallocNumaUser : 0u);
-        const hipError_t allocated = hipHostMalloc(&pointer, rt->z.size_bytes, flags);
-        if (allocated != hipSuccess) {
-            status = set_error(PCIE_EP_E_HIP, "hipHostMalloc of a %zu-byte source segment failed: %s", rt->z.size_bytes, hipGetErrorString(allocated));
-            break;
-        }
-        std::memset(pointer, 0, rt->z.size_bytes);
-        rt->segments[rank] = static_cast<char*>(pointer);
+    if (dims.domains) {
+        int rank_domain[kMaxRanks];
+        numa_domains(*config, rt->domain_node, rank_domain);
     }
-    if (bind) syscall(SYS_set_mempolicy, MPOL_DEFAULT, nullptr, 0);
+    for (int rank = 0; rank < dims.num_ranks && !status; ++rank) {
+        int node = config->staging_numa_node;
+        if (node < 0 && dims.domains && numa_node_exists(config->rank_numa_nodes[rank])) node = config->rank_numa_nodes[rank];
+        status = pinned_zeroed(rt->z.size_bytes, node, &rt->segments[rank], "source segment");
+        for (int domain = 0; domain < dims.domains && !status; ++domain) {
+            const bool present = numa_node_exists(rt->domain_node[domain]);
+            rt->domain_bound[domain] = present;
+            status = pinned_zeroed(rt->z.replica_region_bytes, present ? rt->domain_node[domain] : -1, &rt->replica[rank * kMaxDomains + domain],
+                                   "replica region");
+        }
+    }
     if (!status) {
         const size_t history = size_t(dims.channels) * ((dims.max_tokens + dims.channels - 1) / dims.channels) * 4;
         hipError_t error = hipMalloc(reinterpret_cast<void**>(&rt->epoch), 256);
@@ -401,14 +468,27 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     if (status) {
         for (char* segment : rt->segments)
             if (segment) (void)hipHostFree(segment);
+        for (char* region : rt->replica)
+            if (region) (void)hipHostFree(region);
         if (rt->epoch) (void)hipFree(rt->epoch);
         if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
         if (rt->queues) (void)hipFree(rt->queues);
         if (rt->layout_scratch) (void)hipFree(rt->layout_scratch);
         return status;
     }
+    RelayOptions relay_options;
+    relay_options.workers_per_domain = config->relay_workers_per_numa > 0 ? config->relay_workers_per_numa : 1;
+    relay_options.timeout_ms = config->timeout_ms;
+    relay_options.delay_ns = config->relay_delay_ns;
+    relay_options.cpus.assign(config->relay_cpus, config->relay_cpus + (dims.domains ? config->relay_cpu_count : 0));
+    std::copy(rt->domain_node, rt->domain_node + kMaxDomains, relay_options.domain_node);
+    // This rank's relay workers start before the first dispatch and wait for
+    // epoch 1 (advanced.hpp:113-115).
+    if (dims.domains)
+        rt->relay = std::make_unique<NumaRelay>(rt->z, config->local_rank, rt->segments, rt->replica + config->local_rank * kMaxDomains, relay_options);
     if (config->peer_threads > 0 && dims.num_ranks > 1)
-        rt->peers = std::make_unique<PeerEmulator>(rt->z, config->local_rank, rt->segments, config->peer_threads, config->timeout_ms);
+        rt->peers = std::make_unique<PeerEmulator>(rt->z, config->local_rank, rt->segments, rt->replica, config->peer_threads, config->timeout_ms,
+                                                   relay_options);
     *out = rt.release();
     return 0;
 }
@@ -416,11 +496,19 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
 int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     if (!rt) return 0;
     rt->closed = true;
+    // Tell the relay workers of every rank to stop before their memory goes away
+    // (the reference's destructor raises relay_failed = 199: advanced.hpp:256-262).
+    if (rt->relay) rt->relay->stop_and_join();
     rt->peers.reset();  // joins the emulator threads before the segments go away
+    rt->relay.reset();
     int status = 0;
     for (char*& segment : rt->segments) {
         if (segment && hipHostFree(segment) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a source segment failed");
         segment = nullptr;
+    }
+    for (char*& region : rt->replica) {
+        if (region && hipHostFree(region) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a replica region failed");
+        region = nullptr;
     }
     if (rt->epoch) (void)hipFree(rt->epoch);
     if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
@@ -551,6 +639,60 @@ int pcie_ep_set_test_epoch(pcie_ep_runtime* rt, uint64_t epoch) {
     return 0;
 }
 
+static int page_node(const void* address) {
+    int node = -1;
+    if (syscall(SYS_get_mempolicy, &node, nullptr, 0ul, address, MPOL_F_NODE | MPOL_F_ADDR) != 0) return -errno;
+    return node;
+}
+
+int pcie_ep_relay_diagnostics(pcie_ep_runtime* rt, pcie_ep_relay_summary* summary, pcie_ep_relay_flow* flows, int32_t capacity) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!summary || capacity < 0 || (capacity && !flows)) return set_error(PCIE_EP_E_INVALID, "bad relay diagnostics arguments");
+    static_assert(sizeof(pcie_ep_relay_flow) == sizeof(RelayFlowRecord), "relay flow record layout");
+    std::memset(summary, 0, sizeof *summary);
+    const Dimensions& d = rt->z.dims;
+    summary->enabled = d.domains ? 1 : 0;
+    summary->rank = rt->config.local_rank;
+    summary->num_domains = d.domains;
+    summary->slot_stride = int64_t(rt->z.slot_stride);
+    summary->segment_bytes = int64_t(rt->z.size_bytes);
+    summary->replica_region_bytes = d.domains ? int64_t(rt->z.replica_region_bytes) : 0;
+    for (int rank = 0; rank < kMaxRanks; ++rank) summary->rank_numa_nodes[rank] = rank < d.num_ranks ? rt->config.rank_numa_nodes[rank] : -1;
+    if (!rt->relay) return 0;
+    char* own = rt->segments[rt->config.local_rank];
+    summary->source_page_node = page_node(own + rt->z.slots_offset);
+    for (int domain = 0; domain < d.domains; ++domain) {
+        summary->domain_numa_nodes[domain] = rt->domain_node[domain];
+        summary->domain_bound[domain] = rt->domain_bound[domain] ? 1 : 0;
+        summary->replica_page_node[domain] = page_node(rt->replica[rt->config.local_rank * kMaxDomains + domain]);
+    }
+    summary->workers = rt->relay->workers();
+    summary->flows = rt->relay->flows();
+    summary->epoch = rt->relay->ready_epoch();
+    std::vector<RelayFlowRecord> records(size_t(summary->flows));
+    rt->relay->diagnostics(records.data(), summary->flows);
+    for (int index = 0; index < summary->flows; ++index) {
+        const RelayFlowRecord& r = records[size_t(index)];
+        if (r.epoch == summary->epoch) {
+            summary->copies += r.copied_tokens;
+            summary->payload_bytes += r.copied_payload_bytes;
+        }
+        summary->copies_total += r.copies_total;
+        summary->payload_bytes_total += r.payload_bytes_total;
+        if (index < capacity) std::memcpy(flows + index, &r, sizeof r);
+    }
+    const std::string errors = rt->relay->worker_errors();
+    if (!errors.empty()) return set_error(PCIE_EP_E_PROTOCOL, "relay worker failed: %s", errors.c_str());
+    return 0;
+}
+
+int pcie_ep_set_relay_delay_ns(pcie_ep_runtime* rt, uint64_t delay_ns) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!rt->relay) return set_error(PCIE_EP_E_STATE, "NUMA relay is not enabled");
+    rt->relay->set_delay(delay_ns);
+    return 0;
+}
+
 int pcie_ep_device_numa_node(int32_t device) {
     char bus_id[64] = {};
     if (hipDeviceGetPCIBusId(bus_id, sizeof bus_id, device) != hipSuccess) return -1;
@@ -570,6 +712,8 @@ static uint64_t* host_signal(pcie_ep_runtime* rt, int32_t segment_rank, int32_t 
         case 1: return index >= 0 && index < rt->z.dims.channels ? signal_at(segment, rt->z.channel_abort_offset, index) : nullptr;
         case 2: return signal_at(segment, rt->z.counts_ready_offset);
         case 3: return index >= 0 && index < rt->z.dims.num_ranks ? signal_at(segment, rt->z.counts_consumed_offset, index) : nullptr;
+        case 4: return index >= 0 && index < rt->z.dims.channels * rt->z.dims.domains ? signal_at(segment, rt->z.relay_failed_offset, index) : nullptr;
+        case 5: return index >= 0 && index < rt->z.dims.channels * rt->z.dims.domains ? signal_at(segment, rt->z.relay_drained_offset, index) : nullptr;
         default: return nullptr;
     }
 }

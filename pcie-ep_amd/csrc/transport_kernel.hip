@@ -233,7 +233,8 @@ __device__ bool prepare_receive_prefixes(const DeviceState& state, int lane) {
 // ---------------------------------------------------------------------------------------
 __device__ void tx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
     const SegmentLayout& z = state.z;
-    const int ranks = z.dims.num_ranks, channels = z.dims.channels, me = state.local_rank;
+    const int channels = z.dims.channels, me = state.local_rank;
+    const int endpoints = z.endpoints;  // destination ranks, then (relay mode) one relay endpoint per domain
     const int slots = z.dims.payload_slots;
     const int stride = (z.dims.max_tokens + channels - 1) / channels;
     char* own = state.seg[me];
@@ -246,27 +247,29 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     const uint64_t below = lanes_below(lane);
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
     int produced = 0;
-    int reserved[kMaxRanks];
+    int reserved[kMaxEndpoints];
 #pragma unroll
-    for (int rank = 0; rank < kMaxRanks; ++rank) reserved[rank] = 0;
+    for (int endpoint = 0; endpoint < kMaxEndpoints; ++endpoint) reserved[endpoint] = 0;
     bool failed = false;
     int64_t stage_busy = 0, prepared_ahead = 0;
 
     for (int base = 0; base < candidates && !failed; base += kWave) {
         const int candidate = base + lane;
         const int token = channel + candidate * channels;
-        const uint32_t remote = candidate < candidates ? (state.plan_mask[token] & ~(1u << me)) : 0u;
+        // Where the token is published: its destination ranks, with those of other
+        // domains folded into one relay endpoint per domain (advanced_common.cuh:207-225).
+        const uint32_t remote = candidate < candidates ? endpoint_mask_of(z.dims, me, state.plan_mask[token]) : 0u;
         const uint64_t batch = __ballot(remote != 0);
         if (!batch) continue;
         const int ordinal = produced + __popcll(batch & below);
-        int my_descriptor[kMaxRanks];
+        int my_descriptor[kMaxEndpoints];
 #pragma unroll
-        for (int rank = 0; rank < kMaxRanks; ++rank) {
-            my_descriptor[rank] = 0;
-            if (rank < ranks) {
-                const uint64_t hits = __ballot((remote >> rank) & 1u);
-                my_descriptor[rank] = reserved[rank] + __popcll(hits & below);
-                reserved[rank] += __popcll(hits);
+        for (int endpoint = 0; endpoint < kMaxEndpoints; ++endpoint) {
+            my_descriptor[endpoint] = 0;
+            if (endpoint < endpoints) {
+                const uint64_t hits = __ballot((remote >> endpoint) & 1u);
+                my_descriptor[endpoint] = reserved[endpoint] + __popcll(hits & below);
+                reserved[endpoint] += __popcll(hits);
             }
         }
         // Ring history: which token occupied ordinal i (needed when a slot is reused).
@@ -285,8 +288,8 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
                 device_store_b32(ring, at + 8, remote);
                 device_store_b32(ring, at + 12, uint32_t(channel));
 #pragma unroll
-                for (int rank = 0; rank < kMaxRanks; ++rank)
-                    if (rank < ranks) device_store_b32(ring, at + 16 + 4 * rank, uint32_t(my_descriptor[rank]));
+                for (int endpoint = 0; endpoint < kMaxEndpoints; ++endpoint)
+                    if (endpoint < endpoints) device_store_b32(ring, at + 16 + 4 * endpoint, uint32_t(my_descriptor[endpoint]));
                 // Ring history and the ticket body are complete before the tag.
                 wait_memory_ops();
                 device_store(q.tx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
@@ -314,29 +317,38 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     // slots were checked when they were reused (advanced_dispatch.cuh:229-285).
     // Lanes poll different (ordinal, destination) pairs in parallel.
     bool drained = failed;
+    // Relay mode: every relay flow of the channel, also one without work, must
+    // have consumed this epoch's counts and released its replica slots before a
+    // later dispatch may overwrite the mailbox (advanced_dispatch.cuh:213-225).
+    bool relays_drained = z.dims.domains == 0;
     int drain_ordinal = produced > slots ? produced - slots : 0;
     bool workers_finished = false;
     while (true) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
         if (workers_finished && !drained) {
-            // Each pass checks up to 64 / P ordinals with one lane per destination.
-            const int per_pass = kWave / ranks;
-            const int my_ordinal = drain_ordinal + lane / ranks;
-            const int destination = lane % ranks;
+            // Each pass checks up to 64 / endpoints ordinals with one lane per endpoint.
+            const int per_pass = kWave / endpoints;
+            const int my_ordinal = drain_ordinal + lane / endpoints;
+            const int endpoint = lane % endpoints;
             bool acked = true;
-            if (lane < per_pass * ranks && my_ordinal < produced) {
+            if (lane < per_pass * endpoints && my_ordinal < produced) {
                 const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
-                const uint32_t remote = state.plan_mask[token] & ~(1u << me);
-                if ((remote >> destination) & 1u)
-                    acked = host_load(ack_at(z, own, channel, my_ordinal % slots, destination)) == sequence(epoch, token);
+                const uint32_t remote = endpoint_mask_of(z.dims, me, state.plan_mask[token]);
+                if ((remote >> endpoint) & 1u)
+                    acked = host_load(ack_at(z, own, channel, my_ordinal % slots, endpoint)) == sequence(epoch, token);
             }
             const uint64_t missing = __ballot(!acked);
             if (!missing) drain_ordinal += per_pass;
-            else drain_ordinal += __builtin_ctzll(missing) / ranks;  // everything before the first miss is done
+            else drain_ordinal += __builtin_ctzll(missing) / endpoints;  // everything before the first miss is done
             if (drain_ordinal >= produced) drained = true;
         }
-        if (workers_finished && drained && broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
+        if (workers_finished && drained && !relays_drained) {
+            bool done = true;
+            if (lane < z.dims.domains) done = host_load(signal_at(own, z.relay_drained_offset, flow_index(z, channel, lane))) == epoch;
+            relays_drained = __all(done);
+        }
+        if (workers_finished && drained && (relays_drained || failed) && broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
         // Guardian: this wavefront outlives TX so that a stalled RX still times out.
         const bool unhealthy = health.poll(state, lane);
         const bool forced = channel == 0 && state.control_abort_after && now_ticks() - start >= state.control_abort_after;
@@ -379,6 +391,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
     const int source = lane / lookahead, ahead = lane % lookahead;
     const bool member = source < ranks && source != me;
+    const bool replica = member && reads_replica(z.dims, source, me);
+    const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
     const int expected = member ? state.expected_receive_counts[channel * ranks + source] : 0;
     int total = ahead == 0 ? expected : 0;
     for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
@@ -393,7 +407,11 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
-        Descriptor* descriptor = descriptor_at(z, state.seg[member ? source : me], channel, me, want ? ordinal : 0);
+        // A source of another domain is read from the replica ring its relay fills
+        // for this rank's domain (advanced_common.cuh:237-247).
+        char* segment = state.seg[member ? source : me];
+        Descriptor* descriptor = replica ? replica_descriptor_at(z, segment, channel, my_domain, me, want ? ordinal : 0)
+                                         : descriptor_at(z, segment, channel, me, want ? ordinal : 0);
         // One 16-byte load brings READY together with the slot and token it guards.
         u32x4 published = {0u, 0u, 0u, 0u};
         if (want) published = host_load_b128(host_resource(descriptor, 16), 0);
@@ -423,6 +441,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                 device_store_b32(ring, at + 16, uint32_t(payload_sequence));
                 device_store_b32(ring, at + 20, uint32_t(payload_sequence >> 32));
                 device_store_b32(ring, at + 24, uint32_t(issued + __popcll(accepted & below)));
+                device_store_b32(ring, at + 28, replica ? 1u : 0u);
                 // The ticket body is complete before its tag.
                 wait_memory_ops();
                 device_store(q.rx_ready + ticket_index % kRing, sequence(epoch, ticket_index));
@@ -441,7 +460,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         // store per source for the whole run (entries are consumed in order).  The
         // payload ACK and the ticket ring entry are separate resources.
         if (member && ahead == 0 && run > 0 && !failed)
-            host_field_store(credit_at(z, state.seg[source], channel, me), sequence(epoch, consumed + run - 1));
+            host_field_store(replica ? replica_credit_at(z, state.seg[source], channel, my_domain, me) : credit_at(z, state.seg[source], channel, me),
+                             sequence(epoch, consumed + run - 1));
         if (member) consumed += run;
     }
     // RX is finished when every ticket has been retired by a worker.
@@ -547,6 +567,7 @@ template <bool kFp8, bool kVector>
 __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
+    const int endpoint_count = z.endpoints;
     const int slots = z.dims.payload_slots, descriptors = z.dims.descriptor_slots;
     const int stride = (z.dims.max_tokens + z.dims.channels - 1) / z.dims.channels;
     char* own = state.seg[me];
@@ -554,7 +575,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
     const int meta_dwords = z.meta_bytes / 4;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
     Deadline deadline(now_ticks());
-    int64_t writes = 0, deliveries = 0, credit_miss = 0;
+    int64_t writes = 0, deliveries = 0, published = 0, credit_miss = 0;
     while (true) {
         const int ticket_index = claim_ticket(q.tx_head, lane);
         if (wait_ticket(state, q, q.tx_ready, q.tx_head, ticket_index, epoch, lane, deadline) < 0) break;
@@ -564,22 +585,22 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         const int token = __shfl(int(word), 0), ordinal = __shfl(int(word), 1);
         const uint32_t endpoints = uint32_t(__shfl(int(word), 2));
         const int channel = __shfl(int(word), 3);
-        const int my_descriptor = __shfl(int(word), 4 + (lane < ranks ? lane : 0));
+        const int my_descriptor = __shfl(int(word), 4 + (lane < endpoint_count ? lane : 0));
         wait_memory_ops();
         if (lane == 0) device_store(q.tx_taken + ticket_index % kRing, sequence(epoch, ticket_index));
         const int slot = ordinal % slots;
-        const bool targeted = lane < ranks && ((endpoints >> lane) & 1u);
+        const bool targeted = lane < endpoint_count && ((endpoints >> lane) & 1u);
         if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2] = ticks_to_ns(state, now_ticks());
 
         // Flow control: the slot's previous occupant must be ACKed by all its
         // targets and a descriptor entry must have been consumed before reuse
-        // (advanced_dispatch.cuh:158-187).  One lane per destination.
+        // (advanced_dispatch.cuh:158-187).  One lane per endpoint.
         bool slot_ok = true, credit_ok = true;
         uint64_t previous_sequence = 0;
         if (ordinal >= slots) {
             const int previous_token = device_load(state.chan_remote_tokens + size_t(channel) * stride + ordinal - slots);
-            const uint32_t previous_remote = state.plan_mask[previous_token] & ~(1u << me);
-            slot_ok = !(lane < ranks && ((previous_remote >> lane) & 1u));
+            const uint32_t previous_remote = endpoint_mask_of(z.dims, me, state.plan_mask[previous_token]);
+            slot_ok = !(lane < endpoint_count && ((previous_remote >> lane) & 1u));
             previous_sequence = sequence(epoch, previous_token);
         }
         if (targeted && my_descriptor >= descriptors) credit_ok = false;
@@ -634,7 +655,10 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         }
         if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(state, now_ticks());
         ++writes;
-        deliveries += __popc(endpoints);
+        // Logical deliveries count destination ranks; a relay endpoint stands for
+        // all targeted ranks of its domain with one descriptor.
+        deliveries += __popc(state.plan_mask[token] & ~(1u << me));
+        published += __popc(endpoints);
         fence_lds();  // scratch is reused by the next ticket
         if (lane == 0) device_add(&q.tx_retired[channel].value, 1u);
     }
@@ -644,7 +668,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats);
         atomicAdd(stats + kStatHostWrites, static_cast<unsigned long long>(writes));
         atomicAdd(stats + kStatDeliveries, static_cast<unsigned long long>(deliveries));
-        atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(deliveries));
+        atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(published));
         atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(credit_miss));
     }
 }
@@ -671,11 +695,14 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
         const int channel = __shfl(int(word), 3);
         const uint64_t payload_sequence = uint64_t(uint32_t(__shfl(int(word), 4))) | uint64_t(uint32_t(__shfl(int(word), 5))) << 32;
         const int channel_ordinal = __shfl(int(word), 6);
+        const bool replica = __shfl(int(word), 7) != 0;
         // The ticket now lives in registers: its ring entry may be reused while
         // this wavefront is still moving the row.
         wait_memory_ops();
         if (lane == 0) device_store(q.rx_taken + ticket_index % kRing, sequence(epoch, ticket_index));
-        const char* slot_base = slot_at(z, state.seg[source], channel, slot);
+        const char* slot_base = replica ? replica_slot_at(z, state.replica_in[source], channel, slot) : slot_at(z, state.seg[source], channel, slot);
+        uint64_t* slot_ack = replica ? replica_ack_at(z, state.seg[source], channel, z.dims.rank_domain[me], slot, me)
+                                     : ack_at(z, state.seg[source], channel, slot, me);
         const __amdgpu_buffer_rsrc_t payload = host_resource(slot_base, uint32_t(z.payload_bytes));
         const __amdgpu_buffer_rsrc_t slot_meta = host_resource(slot_base + z.meta_offset, uint32_t(z.meta_bytes));
         if (lane == kWave - 1) test_delay(state.rx_delay);
@@ -781,7 +808,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                 const bool last_pass = first_wire + wire_per_pass >= wire_vectors;
                 if (last_pass) {
                     // All loads of the staged row have returned: release the host slot.
-                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, slot, me), payload_sequence);
+                    if (lane == 0) host_store_release(slot_ack, payload_sequence);
                 }
                 if constexpr (kFp8) {
                     // 16 codes -> 16 BF16 (two 16-byte vectors); expanded in place from the top.
@@ -827,7 +854,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                     }
                 }
                 if (first + kPassScalars * kWave >= hidden) {
-                    if (lane == 0) host_store_release(ack_at(z, state.seg[source], channel, slot, me), payload_sequence);
+                    if (lane == 0) host_store_release(slot_ack, payload_sequence);
                 }
                 uint64_t remaining = destinations;
                 while (remaining) {

@@ -15,6 +15,19 @@
 //  * sizes the per-slot metadata by the runtime top-k instead of 32 branches,
 //  * stores it in the tail of the payload slot so one contiguous region is read,
 //  * groups the count mailbox by destination so a receiver reads one block.
+//
+// Relay mode (csrc/comm/numa_relay.hpp; advanced_common.cuh:207-260).  Ranks
+// are grouped into NUMA domains.  A source reaches a destination of its own
+// domain directly; destinations of another domain n are reached through
+// endpoint P + n: the source publishes ONE descriptor per token to that
+// endpoint, a CPU relay worker of the source copies the slot into the replica
+// ring of domain n (memory bound to that domain's node), publishes replica
+// descriptors to every targeted rank of the domain, and ACKs the source slot.
+// Receivers of domain n read replica slots and answer with replica ACKs and
+// replica credits.  Replica slots, replica descriptors, relay_drained and
+// relay_failed are written only by the source's relay; replica ACKs and replica
+// credits only by the receiver they belong to.  In direct mode there are no
+// domains and none of these regions exist.
 #pragma once
 
 #include <cstddef>
@@ -32,6 +45,8 @@ constexpr int kMaxRanks = 16;      // common.cuh:12
 constexpr int kMaxTopk = 32;       // common.cuh:13
 constexpr int kMaxExperts = 4096;  // common.cuh:14
 constexpr int kMaxChannels = 32;   // pcie_ep/config.py:71
+constexpr int kMaxDomains = 8;     // NUMA domains of a relay configuration (advanced_common.cuh:8)
+constexpr int kMaxEndpoints = kMaxRanks + kMaxDomains;
 constexpr int kErrorFields = 8;
 constexpr int kStatFields = 8;
 constexpr size_t kSignalBytes = 128;  // one writer per 128-byte line
@@ -124,6 +139,9 @@ struct Dimensions {
     int payload_slots;     // Q, per channel
     int descriptor_slots;  // L, per (channel, destination)
     int wire_fp8;          // 0: BF16 payload, 1: E4M3FN payload + FP32 scale
+    int domains;           // N NUMA domains in relay mode, 0 in direct mode
+    int replica_slots;     // R per (channel, domain)
+    int rank_domain[kMaxRanks];  // domain of every rank (relay mode)
 };
 
 struct SegmentLayout {
@@ -144,8 +162,20 @@ struct SegmentLayout {
     size_t ack_offset;              // [C*Q][P] signals
     size_t descriptors_offset;      // [C][P] queues of L packed entries, each queue 128-byte aligned
     size_t descriptor_queue_stride;
-    size_t credits_offset;          // [C][P] signals: sequence(epoch, last ordinal the destination consumed)
+    size_t credits_offset;          // [C][P+N] signals: sequence(epoch, last ordinal the destination consumed)
+    // Relay mode only.
+    int endpoints;                  // P + N
+    size_t relay_mailbox_offset;    // [N] blocks of C dwords: tokens of each channel bound for the domain through the relay
+    size_t relay_mailbox_stride;
+    size_t replica_ack_offset;      // [C][N][R][P] signals
+    size_t replica_descriptors_offset;  // [C][N][P] queues of L packed entries
+    size_t replica_credits_offset;  // [C][N][P] signals
+    size_t relay_drained_offset;    // [C][N] signals: epoch whose flow has been copied and released
+    size_t relay_failed_offset;     // [C][N] signals: non-zero relay failure code
     size_t size_bytes;
+    // Replica payload slots live in one separate region per domain, [C][R] slots
+    // of slot_stride bytes, so that each can be bound to its domain's memory.
+    size_t replica_region_bytes;
 };
 
 // Mailbox block written by source s for destination d:
@@ -172,15 +202,46 @@ PCIE_EP_HD SegmentLayout make_segment_layout(const Dimensions& dims) {
     z.abort_offset = reserve(sizeof(Signal));
     z.channel_abort_offset = reserve(size_t(dims.channels) * sizeof(Signal));
     z.mailbox_offset = reserve(size_t(dims.num_ranks) * z.mailbox_stride);
+    z.endpoints = dims.num_ranks + dims.domains;
+    z.relay_mailbox_stride = align_up(size_t(dims.channels) * 4, kSignalBytes);
+    z.relay_mailbox_offset = reserve(size_t(dims.domains) * z.relay_mailbox_stride);
     cursor = align_up(cursor, kPageBytes);
     const size_t slots = size_t(dims.channels) * dims.payload_slots;
     z.slots_offset = reserve(slots * z.slot_stride);
-    z.ack_offset = reserve(slots * dims.num_ranks * sizeof(Signal));
+    z.ack_offset = reserve(slots * z.endpoints * sizeof(Signal));
     z.descriptor_queue_stride = align_up(size_t(dims.descriptor_slots) * sizeof(Descriptor), kSignalBytes);
-    z.descriptors_offset = reserve(size_t(dims.channels) * dims.num_ranks * z.descriptor_queue_stride);
-    z.credits_offset = reserve(size_t(dims.channels) * dims.num_ranks * sizeof(Signal));
+    z.descriptors_offset = reserve(size_t(dims.channels) * z.endpoints * z.descriptor_queue_stride);
+    z.credits_offset = reserve(size_t(dims.channels) * z.endpoints * sizeof(Signal));
+    const size_t flows = size_t(dims.channels) * dims.domains;
+    z.replica_ack_offset = reserve(flows * dims.replica_slots * dims.num_ranks * sizeof(Signal));
+    z.replica_descriptors_offset = reserve(flows * dims.num_ranks * z.descriptor_queue_stride);
+    z.replica_credits_offset = reserve(flows * dims.num_ranks * sizeof(Signal));
+    z.relay_drained_offset = reserve(flows * sizeof(Signal));
+    z.relay_failed_offset = reserve(flows * sizeof(Signal));
     z.size_bytes = align_up(cursor, kPageBytes);
+    z.replica_region_bytes = align_up(size_t(dims.channels) * dims.replica_slots * z.slot_stride, kPageBytes);
     return z;
+}
+
+// Endpoint through which `source` reaches `destination`: the destination itself
+// inside one domain (or in direct mode), the relay endpoint P + domain otherwise
+// (advanced_common.cuh:207-212).
+PCIE_EP_HD int endpoint_of(const Dimensions& d, int source, int destination) {
+    if (!d.domains || d.rank_domain[source] == d.rank_domain[destination]) return destination;
+    return d.num_ranks + d.rank_domain[destination];
+}
+// Endpoints a token with destination ranks `rank_mask` is published to by `source`.
+PCIE_EP_HD uint32_t endpoint_mask_of(const Dimensions& d, int source, uint32_t rank_mask) {
+    rank_mask &= ~(1u << source);
+    if (!d.domains) return rank_mask;
+    uint32_t endpoints = 0;
+    for (int rank = 0; rank < d.num_ranks; ++rank)
+        if ((rank_mask >> rank) & 1u) endpoints |= 1u << endpoint_of(d, source, rank);
+    return endpoints;
+}
+// Whether `receiver` reads the rows of `source` from a replica ring (advanced_common.cuh:233-235).
+PCIE_EP_HD bool reads_replica(const Dimensions& d, int source, int receiver) {
+    return d.domains && d.rank_domain[source] != d.rank_domain[receiver];
 }
 
 PCIE_EP_HD uint64_t* signal_at(char* segment, size_t offset, size_t index = 0) {
@@ -189,15 +250,35 @@ PCIE_EP_HD uint64_t* signal_at(char* segment, size_t offset, size_t index = 0) {
 PCIE_EP_HD char* slot_at(const SegmentLayout& z, char* segment, int channel, int slot) {
     return segment + z.slots_offset + (size_t(channel) * z.dims.payload_slots + slot) * z.slot_stride;
 }
-PCIE_EP_HD uint64_t* ack_at(const SegmentLayout& z, char* segment, int channel, int slot, int destination) {
-    return signal_at(segment, z.ack_offset, (size_t(channel) * z.dims.payload_slots + slot) * z.dims.num_ranks + destination);
+// `endpoint` is a destination rank or, in relay mode, P + domain.
+PCIE_EP_HD uint64_t* ack_at(const SegmentLayout& z, char* segment, int channel, int slot, int endpoint) {
+    return signal_at(segment, z.ack_offset, (size_t(channel) * z.dims.payload_slots + slot) * z.endpoints + endpoint);
 }
-PCIE_EP_HD Descriptor* descriptor_at(const SegmentLayout& z, char* segment, int channel, int destination, int ordinal) {
-    char* queue = segment + z.descriptors_offset + (size_t(channel) * z.dims.num_ranks + destination) * z.descriptor_queue_stride;
+PCIE_EP_HD Descriptor* descriptor_at(const SegmentLayout& z, char* segment, int channel, int endpoint, int ordinal) {
+    char* queue = segment + z.descriptors_offset + (size_t(channel) * z.endpoints + endpoint) * z.descriptor_queue_stride;
     return reinterpret_cast<Descriptor*>(queue) + ordinal % z.dims.descriptor_slots;
 }
-PCIE_EP_HD uint64_t* credit_at(const SegmentLayout& z, char* segment, int channel, int destination) {
-    return signal_at(segment, z.credits_offset, size_t(channel) * z.dims.num_ranks + destination);
+PCIE_EP_HD uint64_t* credit_at(const SegmentLayout& z, char* segment, int channel, int endpoint) {
+    return signal_at(segment, z.credits_offset, size_t(channel) * z.endpoints + endpoint);
+}
+// Relay mode: replica ring of (channel, domain) inside the segment of the source
+// whose relay fills it; `region` is that source's replica payload region of the domain.
+PCIE_EP_HD size_t flow_index(const SegmentLayout& z, int channel, int domain) { return size_t(channel) * z.dims.domains + domain; }
+PCIE_EP_HD char* replica_slot_at(const SegmentLayout& z, char* region, int channel, int slot) {
+    return region + (size_t(channel) * z.dims.replica_slots + slot) * z.slot_stride;
+}
+PCIE_EP_HD uint64_t* replica_ack_at(const SegmentLayout& z, char* segment, int channel, int domain, int slot, int destination) {
+    return signal_at(segment, z.replica_ack_offset, (flow_index(z, channel, domain) * z.dims.replica_slots + slot) * z.dims.num_ranks + destination);
+}
+PCIE_EP_HD Descriptor* replica_descriptor_at(const SegmentLayout& z, char* segment, int channel, int domain, int destination, int ordinal) {
+    char* queue = segment + z.replica_descriptors_offset + (flow_index(z, channel, domain) * z.dims.num_ranks + destination) * z.descriptor_queue_stride;
+    return reinterpret_cast<Descriptor*>(queue) + ordinal % z.dims.descriptor_slots;
+}
+PCIE_EP_HD uint64_t* replica_credit_at(const SegmentLayout& z, char* segment, int channel, int domain, int destination) {
+    return signal_at(segment, z.replica_credits_offset, flow_index(z, channel, domain) * z.dims.num_ranks + destination);
+}
+PCIE_EP_HD int32_t* relay_mailbox_at(const SegmentLayout& z, char* segment, int domain) {
+    return reinterpret_cast<int32_t*>(segment + z.relay_mailbox_offset + size_t(domain) * z.relay_mailbox_stride);
 }
 // The source may write entry `ordinal` of a queue of L entries once entry
 // `ordinal - L` has been consumed, i.e. once the credit word of this epoch

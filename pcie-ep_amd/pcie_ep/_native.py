@@ -28,8 +28,23 @@ class Sizes(C.Structure):
     _fields_ = [
         ("unique_rows", C.c_int64), ("expanded_rows", C.c_int64), ("plan_bytes", C.c_int64), ("segment_bytes", C.c_int64),
         ("slot_stride", C.c_int64), ("local_experts", C.c_int32), ("payload_bytes", C.c_int32), ("meta_bytes", C.c_int32),
-        ("mailbox_dwords", C.c_int32), ("transport_threads", C.c_int32), ("transport_workgroups", C.c_int32), ("reserved", C.c_int32 * 6),
+        ("mailbox_dwords", C.c_int32), ("transport_threads", C.c_int32), ("transport_workgroups", C.c_int32), ("num_domains", C.c_int32),
+        ("reserved", C.c_int32 * 3), ("replica_region_bytes", C.c_int64),
     ]
+
+
+class RelayFlow(C.Structure):
+    _fields_ = [(name, C.c_int32) for name in ("channel", "numa_domain", "worker", "cpu", "expected_tokens", "error")] + [
+        (name, C.c_uint64) for name in ("epoch", "copied_tokens", "copied_payload_bytes", "copy_time_ns_total",
+                                        "credit_wait_probes_total", "drained_epoch", "copies_total", "payload_bytes_total")]
+
+
+class RelaySummary(C.Structure):
+    _fields_ = [(name, C.c_int32) for name in ("enabled", "rank", "num_domains", "workers", "flows", "source_page_node")] + [
+        ("rank_numa_nodes", C.c_int32 * 16), ("domain_numa_nodes", C.c_int32 * 8), ("domain_bound", C.c_int32 * 8),
+        ("replica_page_node", C.c_int32 * 8)] + [
+        (name, C.c_uint64) for name in ("epoch", "copies", "payload_bytes", "copies_total", "payload_bytes_total")] + [
+        (name, C.c_int64) for name in ("slot_stride", "segment_bytes", "replica_region_bytes")]
 
 
 # Pointer fields of pcie_ep_dispatch_args in declaration order.
@@ -66,6 +81,8 @@ _PROTOTYPES = {
     "pcie_ep_set_test_control_abort_after_ns": (C.c_int, [C.c_void_p, C.c_uint64]),
     "pcie_ep_set_test_skip_counts_ack_source": (C.c_int, [C.c_void_p, C.c_int32]),
     "pcie_ep_set_test_epoch": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "pcie_ep_relay_diagnostics": (C.c_int, [C.c_void_p, C.POINTER(RelaySummary), C.POINTER(RelayFlow), C.c_int32]),
+    "pcie_ep_set_relay_delay_ns": (C.c_int, [C.c_void_p, C.c_uint64]),
     "pcie_ep_device_numa_node": (C.c_int, [C.c_int32]),
     "pcie_ep_host_signal_store": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_uint64]),
     "pcie_ep_host_signal_load": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64)]),

@@ -117,6 +117,7 @@ class HostStagedEPBuffer:
         tx_waves: int = 0,
         rx_waves: int = 0,
         worker_groups: int = 0,
+        rank_numa_nodes: Optional[Tuple[int, ...]] = None,
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
@@ -131,6 +132,10 @@ class HostStagedEPBuffer:
         shape the transport kernel (0 = defaults: 48 payload workgroups of 2 TX +
         2 RX wavefronts; 64 of 2 TX + 4 RX on the FP8 wire; ``worker_groups=-1`` makes the
         per-channel control workgroups move the rows themselves).
+        ``rank_numa_nodes`` (relay mode) gives the NUMA node of every logical rank,
+        which the reference gathers from its processes; ranks of another node than
+        a source's are reached through that source's relay workers and replica
+        rings.  Default: every rank on the GPU's node, i.e. one domain.
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -170,9 +175,15 @@ class HostStagedEPBuffer:
         self._ordering = _Ordering(self.device)
         self.runtime: Optional[NativeRuntime] = None
         threads = min(num_ranks - 1, 7) if peer_threads is None else peer_threads
+        if rank_numa_nodes is not None:
+            if self.config.numa_mode != "relay":
+                raise ValueError("rank_numa_nodes is meaningful only with numa_mode='relay'")
+            if len(rank_numa_nodes) != num_ranks or any(not isinstance(node, int) or node < -1 for node in rank_numa_nodes):
+                raise ValueError("rank_numa_nodes must name one NUMA node (or -1) per rank")
         self.runtime = NativeRuntime(rank, num_ranks, num_max_tokens_per_rank, hidden, num_topk, num_experts, self.config,
                                      self.device, peer_threads=threads, staging_numa_node=staging_numa_node,
-                                     tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups)
+                                     tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups,
+                                     rank_numa_nodes=rank_numa_nodes)
         self.peers = PeerGroup(self.runtime) if threads > 0 and num_ranks > 1 else None
 
     def _refuse_unsupported_world(self, group: Any, control_group: Any, reuse_comm: bool) -> None:
@@ -186,8 +197,6 @@ class HostStagedEPBuffer:
                 )
         if reuse_comm:
             raise RuntimeError("No NCCL/RCCL communicator is available to borrow in the single-process build")
-        if self.config.numa_mode == "relay":
-            raise NotImplementedError("NUMA relay workers are not part of this build; use numa_mode='direct'")
 
     # ---- streams ------------------------------------------------------------------------
     def get_comm_stream(self) -> Any:

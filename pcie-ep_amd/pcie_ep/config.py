@@ -6,9 +6,11 @@ exception type and message, are the reference's public contract
 sites and configuration files keep working.  Options that only choose between
 code paths of the reference that this build does not have are accepted,
 recorded and ignored where results do not depend on them
-(``receive_expand_mode``, ``pipeline_stages``, ``source_fusion``,
-``warp_specialization``, ``replica_slots``), and rejected at buffer construction
-where they would (``numa_mode='relay'``).
+(``pipeline_stages``, ``source_fusion``, ``warp_specialization``;
+``receive_expand_mode`` only selects what the ``receive_expand_overlap``
+diagnostic holds).  ``numa_mode='relay'`` with ``replica_slots``,
+``relay_workers_per_numa`` and ``relay_cpu_affinity`` starts this rank's CPU relay
+workers (csrc/comm/numa_relay.hpp).
 
 The rejection rules are kept as a table (``_RULES``), evaluated in order: each
 entry is a predicate over the config that is true when the config is *bad*, the
@@ -73,7 +75,7 @@ class HostStagedConfig:
     capacities: they bound what is in flight, not the tokens of one dispatch.
     ``stage`` is a capability gate: 6 = BF16 wire, 7 adds the FP8 wire
     (``wire_dtype='fp8_e4m3'``: E4M3FN bytes plus one FP32 scale per token on
-    the wire, BF16 tensors on both sides), 8 is accepted for compatibility.
+    the wire, BF16 tensors on both sides), 8 adds the NUMA relay (``numa_mode='relay'``).
     """
 
     payload_slots: int = 256

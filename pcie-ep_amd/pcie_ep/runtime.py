@@ -73,7 +73,7 @@ class NativeRuntime:
 
     def __init__(self, rank: int, world: int, max_tokens: int, hidden: int, topk: int, experts: int, config: HostStagedConfig,
                  device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0,
-                 worker_groups: int = 0) -> None:
+                 worker_groups: int = 0, rank_numa_nodes: Optional[tuple] = None) -> None:
         self._lib = _native.library()
         self.config = config
         self.device = torch.device("cuda", device)
@@ -86,7 +86,19 @@ class NativeRuntime:
             peer_threads=peer_threads, staging_numa_node=staging_numa_node, device=device,
             worker_groups=worker_groups,
             receive_expand_mode=("pipelined", "vectorized", "scalar").index(config.receive_expand_mode),
+            numa_mode=int(config.numa_mode == "relay"), replica_slots=config.replica_slots,
+            relay_workers_per_numa=config.relay_workers_per_numa, relay_cpu_count=len(config.relay_cpu_affinity),
         )
+        if len(config.relay_cpu_affinity) > 64:
+            raise ValueError("relay_cpu_affinity holds more than 64 CPUs")
+        for index, cpu in enumerate(config.relay_cpu_affinity):
+            native.relay_cpus[index] = cpu
+        nodes = tuple(rank_numa_nodes) if rank_numa_nodes is not None else (-1,) * world
+        if len(nodes) != world:
+            raise RuntimeError("rank_numa_nodes length differs from EP size")
+        for index in range(16):
+            native.rank_numa_nodes[index] = int(nodes[index]) if index < world else -1
+        self.rank_numa_nodes = nodes
         self.native_config = native
         self.sizes = _native.Sizes()
         _native.check(self._lib.pcie_ep_query_sizes(C.byref(native), C.byref(self.sizes)), invalid=RuntimeError)
@@ -230,6 +242,55 @@ class NativeRuntime:
         value = C.c_uint64()
         _native.check(self._lib.pcie_ep_host_signal_load(self._require(), segment_rank, which, index, C.byref(value)))
         return int(value.value)
+
+    def set_relay_delay_ns(self, delay_ns: int) -> None:
+        """Test hook of the relay workers (``AdvancedRuntime.set_relay_delay_ns``)."""
+        _native.check(self._lib.pcie_ep_set_relay_delay_ns(self._require(), delay_ns), invalid=RuntimeError)
+
+    def relay_diagnostics(self) -> Dict[str, Any]:
+        """State of this rank's NUMA relay workers, shaped like the reference's
+        ``AdvancedRuntime.relay_diagnostics`` (csrc/buffers/advanced.hpp:182-213;
+        csrc/comm/numa_relay.hpp:133-175): per-epoch and total copy counts, one
+        record per worker with its (channel, domain) flows, the NUMA map and where
+        sampled payload pages reside."""
+        summary = _native.RelaySummary()
+        capacity = self.channels * 8
+        flows = (_native.RelayFlow * capacity)()
+        _native.check(self._lib.pcie_ep_relay_diagnostics(self._require(), C.byref(summary), flows, capacity), invalid=RuntimeError)
+        domains = int(summary.num_domains)
+        result: Dict[str, Any] = {
+            "enabled": bool(summary.enabled), "rank": int(summary.rank),
+            "rank_numa_nodes": [int(node) for node in summary.rank_numa_nodes[: self.world]],
+            "physical_numa_nodes": [int(node) for node in summary.domain_numa_nodes[:domains]],
+            "payload_stride_bytes": int(summary.slot_stride), "segment_bytes": int(summary.segment_bytes),
+            "replica_region_bytes": int(summary.replica_region_bytes),
+            "wire_dtype": "fp8_e4m3" if self.config.wire_dtype == "fp8_e4m3" else "bf16",
+            "cpu_handshake": "std::atomic_ref<uint64_t> lock-free acquire/release load/store",
+        }
+        if not summary.enabled:
+            return result
+        workers: Dict[int, Dict[str, Any]] = {}
+        for flow in flows[: min(capacity, int(summary.flows))]:
+            worker = workers.setdefault(int(flow.worker), {
+                "numa_domain": int(flow.numa_domain), "numa_node": int(summary.domain_numa_nodes[flow.numa_domain]),
+                "cpu": int(flow.cpu), "runtime_error": "", "flows": []})
+            worker["flows"].append({
+                "channel": int(flow.channel), "epoch": int(flow.epoch), "expected_tokens": int(flow.expected_tokens),
+                "copied_tokens": int(flow.copied_tokens), "copied_payload_bytes": int(flow.copied_payload_bytes),
+                "copy_time_ns_total": int(flow.copy_time_ns_total), "credit_wait_probes_total": int(flow.credit_wait_probes_total),
+                "drained_epoch": int(flow.drained_epoch), "error": int(flow.error)})
+        result.update({
+            "epoch": int(summary.epoch), "copies": int(summary.copies), "payload_bytes": int(summary.payload_bytes),
+            "copies_total": int(summary.copies_total), "payload_bytes_total": int(summary.payload_bytes_total),
+            "host_read_write_bytes": int(summary.payload_bytes) * 2, "workers": [workers[index] for index in sorted(workers)],
+            "metadata_and_scales_excluded_from_payload_bytes": True,
+            "source_payload_placement": {"sampled_node": int(summary.source_page_node)},
+            "replica_payload_placement": [
+                {"domain": domain, "target_numa_node": int(summary.domain_numa_nodes[domain]), "bound": bool(summary.domain_bound[domain]),
+                 "sampled_node": int(summary.replica_page_node[domain])} for domain in range(domains)],
+            "control_placement": "source NUMA; only replica payload pages are target-bound",
+        })
+        return result
 
     def expand_unique(self, pool_tensors: Dict[str, torch.Tensor], plan: RoutePlan, alignment: int, zero_padding: bool) -> None:
         """Run only the stand-alone expand kernel on an existing result (benchmarks)."""

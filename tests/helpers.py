@@ -137,14 +137,15 @@ def _rows_equal(recv_x: torch.Tensor, out_rows: np.ndarray, bank: torch.Tensor, 
 
 
 def verify_dispatch(result, inputs: Sequence[Inputs], rank: int, world: int, experts: int, topk: int, expand: bool, alignment: int,
-                    zero_padding: bool, with_weights: bool = True, fp8_wire: bool = False, check_stats: bool = True) -> dict:
+                    zero_padding: bool, with_weights: bool = True, fp8_wire: bool = False, check_stats: bool = True,
+                    rank_numa_nodes=None) -> dict:
     recv_x, recv_idx, recv_weights, handle, event = result
     event.current_stream_wait()
     torch.cuda.synchronize()
     error = handle.error.cpu().tolist()
     assert not any(error), f"GPU error {error}"
     all_idx = [idx.numpy() for _, idx, _ in inputs]
-    expectation = oracle.expected_dispatch(all_idx, rank, world, experts, alignment)
+    expectation = oracle.expected_dispatch(all_idx, rank, world, experts, alignment, rank_numa_nodes)
     receiver = expectation.receiver
     assert int(handle.unique_count.cpu()) == receiver.unique_count
     assert int(handle.expanded_count.cpu()) == receiver.expanded_count

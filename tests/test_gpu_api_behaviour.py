@@ -83,8 +83,10 @@ def test_constructor_rejections():
         HostStagedEPBuffer(None, 8, 0, 2, 16)
     with pytest.raises(ValueError, match="uniformly divisible"):
         HostStagedEPBuffer(None, 8, 64, 2, 20)
-    with pytest.raises(NotImplementedError, match="NUMA relay"):
-        HostStagedEPBuffer(None, 8, 64, 2, 16, HostStagedConfig(stage=8, numa_mode="relay"))
+    with pytest.raises(ValueError, match="only with numa_mode='relay'"):
+        HostStagedEPBuffer(None, 8, 64, 2, 16, rank_numa_nodes=(0,) * 8)
+    with pytest.raises(ValueError, match="one NUMA node"):
+        HostStagedEPBuffer(None, 8, 64, 2, 16, HostStagedConfig(stage=8, numa_mode="relay"), rank_numa_nodes=(0, 1))
     with pytest.raises(RuntimeError, match="communicator"):
         HostStagedEPBuffer(None, 8, 64, 2, 16, require_reuse_nccl_comm=True)
     with pytest.raises(RuntimeError, match="unsupported advanced dimensions"):

@@ -268,3 +268,32 @@ def test_cpu_plumbing_configuration_all_eight_receivers():
     assert len(seen) == world * tokens * topk  # nothing lost, nothing duplicated
     volume = oracle.route_volume(idx, world, experts)
     assert total_unique == volume["remote_deliveries"] + sum(int(np.any(idx[r] // local == r, axis=1).sum()) for r in range(world))
+
+
+def test_relay_descriptor_and_copy_counts_against_brute_force():
+    """Relay mode publishes one descriptor per destination of the source's own
+    domain plus one per other domain reached, and the relay copies a row once
+    per other domain (tests/test_relay.py:16-22 of the reference).  Checked
+    against nested loops on random routes; without a NUMA map the counts reduce
+    to one descriptor per delivery and no copies."""
+    rng = np.random.default_rng(11)
+    for world, experts, topk, nodes in [(8, 64, 6, (0, 0, 0, 0, 1, 1, 1, 1)), (6, 24, 4, (2, 0, 1, 1, -1, 2)), (4, 16, 3, (5, 5, 5, 5))]:
+        local = experts // world
+        idx = np.stack([rng.permutation(experts)[:topk] for _ in range(97)]).astype(np.int64)
+        idx[::5, 0] = -1
+        known = sorted({n for n in nodes if n >= 0})
+        domain = [known.index(n) if n >= 0 else 0 for n in nodes]
+        assert oracle.numa_domains(nodes) == domain
+        for own in range(world):
+            descriptors = copies = deliveries = 0
+            for token in idx:
+                ranks = {int(e) // local for e in token if e >= 0} - {own}
+                deliveries += len(ranks)
+                others = {domain[r] for r in ranks if domain[r] != domain[own]}
+                descriptors += sum(1 for r in ranks if domain[r] == domain[own]) + len(others)
+                copies += len(others)
+            layout = oracle.source_layout(idx, world, experts)
+            relay = layout.source_statistics(own, nodes)
+            assert (relay["descriptors_published"], relay["relay_copies"], relay["remote_deliveries"]) == (descriptors, copies, deliveries)
+            direct = layout.source_statistics(own)
+            assert direct["descriptors_published"] == deliveries and direct["relay_copies"] == 0
