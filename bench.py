@@ -180,7 +180,20 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
         mean_ms = sum(durations) / len(durations)
         algorithmic = (unique + expanded) * HIDDEN * 2 + expanded * 36
         del result, handle
+        # The same traffic shape with no metadata and no dependent loads (one row
+        # read, one written, the same share of rows written twice), by write order:
+        # what HBM gives a write-heavy row scatter on this part.
+        from pcie_ep import _native
+
+        ceilings = {}
+        extra = max(0, min(1024, round((expanded / max(unique, 1) - 1.0) * 1024)))
+        for name, pattern in (("linear", 0), ("expert_streams", 1), ("hashed", 2)):
+            rate = _native.C.c_double()
+            _native.check(_native.library().pcie_ep_measure_row_scatter(0, unique, HIDDEN * 2, extra, pattern, EXPERTS // WORLD, 5, _native.C.byref(rate)),
+                          invalid=RuntimeError)
+            ceilings[name] = rate.value
         return {
+            "shape_ceiling_GBps": ceilings,
             "bound": "hbm", "kernel": "expand_kernel", "achieved": algorithmic / mean_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": algorithmic / mean_ms / 1e6 / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": algorithmic,
             "avg_us": mean_ms * 1e3, "min_us": min(durations) * 1e3, "unique_rows": unique, "expanded_rows": expanded,

@@ -151,6 +151,36 @@ __global__ void __launch_bounds__(kRowKernelThreads) zero_kernel(u32x4* destinat
         destination[index] = zero;
 }
 
+// Calibration of the expand kernel's traffic SHAPE: every wavefront reads one row
+// and writes it once, and a given fraction of the rows twice, with no metadata
+// and no dependent loads.  The destination order is linear, `streams`
+// interleaved sequential streams (what expert-major placement of source-ordered
+// rows produces), or hashed.  What this reaches is the practical HBM ceiling
+// for a write-heavy row scatter; the expand kernel is compared with it.
+__global__ void __launch_bounds__(kRowKernelThreads) row_scatter_kernel(const u32x4* source, u32x4* destination, int rows, int row_vectors,
+                                                                         int extra_per_1024, int pattern, int streams) {
+    const int lane = threadIdx.x % kWave;
+    const int waves_per_block = blockDim.x / kWave;
+    const int total_waves = gridDim.x * waves_per_block;
+    for (int row = blockIdx.x * waves_per_block + threadIdx.x / kWave; row < rows; row += total_waves) {
+        int out = row;
+        if (pattern == 1) {
+            const int stream = row % streams, position = row / streams, per_stream = rows / streams;
+            if (position < per_stream) out = stream * per_stream + position;
+        } else if (pattern == 2) {
+            out = int(uint64_t(row) * 2654435761ull % uint64_t(rows));
+        }
+        const u32x4* from = source + size_t(row) * row_vectors;
+        for (int first = 0; first < row_vectors; first += kPassItems * kWave) {
+            RowVectors pass;
+            row_load_vectors<true>(pass, from, first, row_vectors, lane);
+            row_store_vectors<true>(pass, destination + size_t(out) * row_vectors, first, row_vectors, lane);
+            if ((row & 1023) * extra_per_1024 / 1024 != ((row & 1023) + 1) * extra_per_1024 / 1024)
+                row_store_vectors<true>(pass, destination + size_t(rows + out) * row_vectors, first, row_vectors, lane);
+        }
+    }
+}
+
 int row_grid(int64_t rows, int64_t cap = 8192) {
     // Four wavefronts per workgroup, one row per wavefront, capped so that the
     // grid-stride loop still spreads over all 256 CUs several times.
@@ -177,6 +207,16 @@ hipError_t launch_zero(void* destination, size_t bytes, hipStream_t stream) {
     if (!vectors) return hipSuccess;
     const size_t blocks = (vectors + kRowKernelThreads - 1) / kRowKernelThreads;
     hipLaunchKernelGGL(zero_kernel, dim3(unsigned(blocks < 1024 ? blocks : 1024)), dim3(kRowKernelThreads), 0, stream, static_cast<u32x4*>(destination), vectors);
+    return hipGetLastError();
+}
+
+hipError_t launch_row_scatter(const void* source, void* destination, int rows, int row_bytes, int extra_per_1024, int pattern, int streams,
+                              hipStream_t stream) {
+    if (rows <= 0 || row_bytes <= 0 || row_bytes % 16 || extra_per_1024 < 0 || extra_per_1024 > 1024 || pattern < 0 || pattern > 2 || streams < 1)
+        return hipErrorInvalidValue;
+    const dim3 grid(row_grid(rows, 16384)), block(kRowKernelThreads);
+    hipLaunchKernelGGL(row_scatter_kernel, grid, block, 0, stream, static_cast<const u32x4*>(source), static_cast<u32x4*>(destination), rows,
+                       row_bytes / 16, extra_per_1024, pattern, streams);
     return hipGetLastError();
 }
 

@@ -856,6 +856,48 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
     return 0;
 }
 
+int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes, int32_t extra_per_1024, int32_t pattern, int32_t streams,
+                                int32_t repeats, double* gbps) {
+    if (rows < 1 || row_bytes < 16 || row_bytes % 16 || extra_per_1024 < 0 || extra_per_1024 > 1024 || pattern < 0 || pattern > 2 || streams < 1 ||
+        repeats < 1 || !gbps)
+        return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
+    HIP_TRY(hipSetDevice(device));
+    const size_t bytes = size_t(rows) * size_t(row_bytes);
+    void *source = nullptr, *destination = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t begin = nullptr, end = nullptr;
+    hipError_t status = hipMalloc(&source, bytes);
+    if (status == hipSuccess) status = hipMalloc(&destination, 2 * bytes);
+    if (status == hipSuccess) status = hipMemset(source, 1, bytes);
+    if (status == hipSuccess) status = hipStreamCreate(&stream);
+    if (status == hipSuccess) status = hipEventCreate(&begin);
+    if (status == hipSuccess) status = hipEventCreate(&end);
+    // Rows written twice, counted exactly as the kernel selects them.
+    int64_t twice = 0;
+    for (int row = 0; row < rows; ++row) twice += (row & 1023) * extra_per_1024 / 1024 != ((row & 1023) + 1) * extra_per_1024 / 1024;
+    double best = 0.0;
+    for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+        status = hipEventRecord(begin, stream);
+        if (status == hipSuccess) status = launch_row_scatter(source, destination, rows, row_bytes, extra_per_1024, pattern, streams, stream);
+        if (status == hipSuccess) status = hipEventRecord(end, stream);
+        if (status == hipSuccess) status = hipEventSynchronize(end);
+        float ms = 0.0f;
+        if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
+        if (status == hipSuccess && i > 0 && ms > 0.0f) {
+            const double rate = double(2 * int64_t(rows) + twice) * double(row_bytes) / (ms * 1e6);  // bytes read + bytes written
+            if (rate > best) best = rate;
+        }
+    }
+    if (begin) (void)hipEventDestroy(begin);
+    if (end) (void)hipEventDestroy(end);
+    if (stream) (void)hipStreamDestroy(stream);
+    if (source) (void)hipFree(source);
+    if (destination) (void)hipFree(destination);
+    if (status != hipSuccess) return set_error(PCIE_EP_E_HIP, "row scatter measurement failed: %s", hipGetErrorString(status));
+    *gbps = best;
+    return 0;
+}
+
 // ---- peer emulator -----------------------------------------------------------------
 
 #define NEED_PEERS(rt)                                                                                        \

@@ -563,8 +563,16 @@ __device__ float tx_copy_row(const DeviceState& state, const uint16_t* input, __
     return 1.0f;
 }
 
+// Counters a payload wavefront accumulates over the rows it moves, flushed once when it ends.
+struct WorkerCounters {
+    int64_t writes = 0, deliveries = 0, published = 0, credit_miss = 0, reads = 0;
+};
+
+// Moves the own token of transmit ticket `ticket_index` (already marked ready)
+// into its host slot and publishes it.  Returns false when the wavefront must stop.
 template <bool kFp8, bool kVector>
-__device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane) {
+__device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, const Deadline& deadline,
+                       WorkerCounters& counters) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
     const int endpoint_count = z.endpoints;
@@ -574,11 +582,7 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
     const uint64_t epoch = *state.epoch;
     const int meta_dwords = z.meta_bytes / 4;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
-    Deadline deadline(now_ticks());
-    int64_t writes = 0, deliveries = 0, published = 0, credit_miss = 0;
-    while (true) {
-        const int ticket_index = claim_ticket(q.tx_head, lane);
-        if (wait_ticket(state, q, q.tx_ready, q.tx_head, ticket_index, epoch, lane, deadline) < 0) break;
+    {
         // Copy the ticket out of the ring (one dword per lane), then free its entry.
         const uint32_t entry_base = uint32_t(ticket_index % kRing) * uint32_t(sizeof(TxEntry));
         const uint32_t word = device_load_b32(ring, entry_base + uint32_t(lane < int(sizeof(TxEntry) / 4) ? lane : 0) * 4u);
@@ -609,14 +613,14 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
             if (!slot_ok) slot_ok = host_load(ack_at(z, own, channel, slot, lane)) == previous_sequence;
             if (!credit_ok) credit_ok = credit_covers(host_load(credit_at(z, own, channel, lane)), epoch, my_descriptor, descriptors);
             if (__all(slot_ok && credit_ok)) break;
-            ++credit_miss;
+            ++counters.credit_miss;
             if (broadcast_first((aborted(q) || deadline.expired(state)) ? 1 : 0)) {
                 stop = true;
                 break;
             }
             backoff();
         }
-        if (stop) break;
+        if (stop) return false;
         compiler_barrier();
 
         // Slot metadata: composed in this wavefront's LDS scratch, then copied out
@@ -654,41 +658,32 @@ __device__ void tx_worker(const DeviceState& state, TransportQueues& q, uint32_t
             host_store_b128(host_resource(descriptor_at(z, own, channel, lane, my_descriptor), 16), 0, entry);
         }
         if (ordinal == 0 && lane == 0) state.prefix_tx_timestamps_ns[(channel + 1) * 2 + 1] = ticks_to_ns(state, now_ticks());
-        ++writes;
+        ++counters.writes;
         // Logical deliveries count destination ranks; a relay endpoint stands for
         // all targeted ranks of its domain with one descriptor.
-        deliveries += __popc(state.plan_mask[token] & ~(1u << me));
-        published += __popc(endpoints);
+        counters.deliveries += __popc(state.plan_mask[token] & ~(1u << me));
+        counters.published += __popc(endpoints);
         fence_lds();  // scratch is reused by the next ticket
         if (lane == 0) device_add(&q.tx_retired[channel].value, 1u);
     }
-    // Workers serve every channel; their counts go to channel 0's row of the
-    // per-channel statistics, whose column sums are what callers read.
-    if (lane == 0 && (writes || credit_miss)) {
-        auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats);
-        atomicAdd(stats + kStatHostWrites, static_cast<unsigned long long>(writes));
-        atomicAdd(stats + kStatDeliveries, static_cast<unsigned long long>(deliveries));
-        atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(published));
-        atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(credit_miss));
-    }
+    return true;
 }
 
 // ---------------------------------------------------------------------------------------
 // RX + scatter worker
 // ---------------------------------------------------------------------------------------
+// Reads the row of receive ticket `ticket_index` (already marked ready) from its
+// host slot and stores it to its destination rows.  Returns false when the
+// wavefront must stop.
 template <bool kFp8, bool kVector>
-__device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane) {
+__device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
     const uint64_t epoch = *state.epoch;
     const bool scatter = state.expand && state.fuse_expand;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
-    Deadline deadline(now_ticks());
-    int64_t reads = 0;
-    while (true) {
-        const int ticket_index = claim_ticket(q.rx_head, lane);
-        if (wait_ticket(state, q, q.rx_ready, q.rx_head, ticket_index, epoch, lane, deadline) < 0) break;
+    {
         const uint32_t entry_base = uint32_t(ticket_index % kRing) * uint32_t(sizeof(RxEntry));
         const uint32_t word = device_load_b32(ring, entry_base + uint32_t(lane < 8 ? lane : 0) * 4u);
         const int source = __shfl(int(word), 0), slot = __shfl(int(word), 1), ticket_token = __shfl(int(word), 2);
@@ -742,7 +737,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                 record_error(state, kErrPayloadSequence);
                 raise_abort(q);
             }
-            break;
+            return false;
         }
 
         // Destination rows, one lane per branch.  Everything the row numbers are
@@ -779,7 +774,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                 record_error(state, kErrPayloadSequence);
                 raise_abort(q);
             }
-            break;
+            return false;
         }
         const int64_t capacity = scatter ? state.expanded_capacity : unique_capacity(z.dims);
         if (__any(my_row >= capacity)) {
@@ -787,7 +782,7 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                 record_error(state, kErrExpandedCapacity);
                 raise_abort(q);
             }
-            break;
+            return false;
         }
         const uint64_t destinations = __ballot(my_row >= 0);
         uint16_t* output_base = scatter ? state.expanded_payload : state.unique_payload;
@@ -895,12 +890,83 @@ __device__ void rx_worker(const DeviceState& state, TransportQueues& q, uint32_t
                 state.unique_source_meta[out_row * 3 + 2] = -1;
             }
         }
-        ++reads;
+        ++counters.reads;
         fence_lds();  // scratch is reused by the next ticket
         if (lane == 0) device_add(&q.rx_retired[channel].value, 1u);
     }
-    if (lane == 0 && reads)
-        atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + kStatHostReads), static_cast<unsigned long long>(reads));
+    return true;
+}
+
+// ---------------------------------------------------------------------------------------
+// Payload wavefront: moves rows of either direction
+// ---------------------------------------------------------------------------------------
+// Every payload wavefront has a home direction (the first tx_waves wavefronts of
+// a workgroup transmit, the others receive) and serves it until every ticket of
+// that direction has been claimed.  Then, instead of leaving, it takes tickets
+// of the other direction: the two directions end together whatever the
+// routing's send/receive ratio is, and the split only sets how the link is shared
+// while both have work.  A ticket of the other direction is only claimed when
+// its producer has already reserved it (head < tail), so a wavefront never
+// commits itself to a row that does not exist yet.
+template <bool kFp8, bool kVector>
+__device__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, bool home_tx) {
+    const uint64_t epoch = *state.epoch;
+    Deadline deadline(now_ticks());
+    WorkerCounters counters;
+    while (true) {
+        // 0: nothing to do now, 1: transmit, 2: receive, -1: both directions are finished or the kernel aborts.
+        int choice = 0;
+        if (lane == 0) {
+            if (aborted(q)) choice = -1;
+            else {
+                const int tx_head = int(device_load(&q.tx_head.value)), rx_head = int(device_load(&q.rx_head.value));
+                const bool tx_backlog = tx_head < int(device_load(&q.tx_tail.value));
+                const bool rx_backlog = rx_head < int(device_load(&q.rx_tail.value));
+                const int tx_total = device_load(&q.tx_head.total), rx_total = device_load(&q.rx_head.total);
+                const bool tx_done = tx_total >= 0 && tx_head >= tx_total, rx_done = rx_total >= 0 && rx_head >= rx_total;
+                if (home_tx ? tx_backlog : rx_backlog) choice = home_tx ? 1 : 2;
+                else if ((home_tx ? tx_done : rx_done) && (home_tx ? rx_backlog : tx_backlog)) choice = home_tx ? 2 : 1;
+                else {
+                    if (tx_done && rx_done) choice = -1;
+                    else if (deadline.expired(state)) {
+                        record_error(state, kErrRingProgressWait);
+                        raise_abort(q);
+                        choice = -1;
+                    }
+                }
+            }
+        }
+        choice = broadcast_first(choice);
+        if (choice < 0) break;
+        if (choice == 0) {
+            backoff();
+            continue;
+        }
+        const bool transmit = choice == 1;
+        QueueCounter& head = transmit ? q.tx_head : q.rx_head;
+        const int ticket_index = claim_ticket(head, lane);
+        // Several wavefronts may have seen the same backlog: a claim beyond the last
+        // ticket of the dispatch is simply dropped, an earlier one waits for its tag.
+        if (wait_ticket(state, q, transmit ? q.tx_ready : q.rx_ready, head, ticket_index, epoch, lane, deadline) < 0) {
+            if (broadcast_first(aborted(q) ? 1 : 0)) break;
+            continue;
+        }
+        const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters)
+                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters);
+        if (!go_on) break;
+    }
+    // Workers serve every channel; their counts go to channel 0's row of the
+    // per-channel statistics, whose column sums are what callers read.
+    if (lane == 0) {
+        auto* stats = reinterpret_cast<unsigned long long*>(state.channel_stats);
+        if (counters.writes || counters.credit_miss) {
+            atomicAdd(stats + kStatHostWrites, static_cast<unsigned long long>(counters.writes));
+            atomicAdd(stats + kStatDeliveries, static_cast<unsigned long long>(counters.deliveries));
+            atomicAdd(stats + kStatDescriptors, static_cast<unsigned long long>(counters.published));
+            atomicAdd(stats + kStatTxCreditMiss, static_cast<unsigned long long>(counters.credit_miss));
+        }
+        if (counters.reads) atomicAdd(stats + kStatHostReads, static_cast<unsigned long long>(counters.reads));
+    }
 }
 
 // Workgroup b < C is the control workgroup of channel b (wavefront 0 TX control,
@@ -935,8 +1001,7 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
         wave -= 2;
     }
     if (wave >= payload_waves) return;
-    if (wave < state.tx_waves) tx_worker<kFp8, kVector>(state, q, scratch, lane);
-    else rx_worker<kFp8, kVector>(state, q, scratch, lane);
+    payload_worker<kFp8, kVector>(state, q, scratch, lane, wave < state.tx_waves);
     finish_role(state, q, lane, roles);
     // Every role loop has an explicit completion, abort or timeout exit and no
     // workgroup barrier follows the entry verdict.

@@ -93,6 +93,7 @@ _PROTOTYPES = {
     "pcie_ep_measure_pinned_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "pcie_ep_measure_kernel_host_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "pcie_ep_measure_device_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double)]),
+    "pcie_ep_measure_row_scatter": (C.c_int, [C.c_int32] * 7 + [C.POINTER(C.c_double)]),
     "pcie_ep_peer_set_source": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
     "pcie_ep_peers_start": (C.c_int, [C.c_void_p, C.c_int32, C.c_uint32]),
     "pcie_ep_peers_wait_staged": (C.c_int, [C.c_void_p, C.c_int32]),
