@@ -49,6 +49,8 @@ class _Ordering:
         self.device = device
         self.stream = torch.cuda.Stream(device=device)
         self.stream.wait_stream(torch.cuda.current_stream(device))
+        self._stream_key = self._key(self.stream)
+        self.raw_stream = int(self.stream.cuda_stream)
         self._consumers: Dict[Tuple[int, int], Any] = {}
         self._guard = threading.Lock()
 
@@ -61,7 +63,7 @@ class _Ordering:
         result pools only behind that stream's tail, even when the Python tensors
         are gone by then (the protection of pcie_ep/buffers/ep.py:197-220)."""
         key = self._key(stream)
-        if key != self._key(self.stream):
+        if key != self._stream_key:
             with self._guard:
                 self._consumers[key] = stream
 
@@ -69,28 +71,40 @@ class _Ordering:
         with self._guard:
             self._consumers.clear()
 
-    def submit(self, work: Callable[[], Any], previous_event: Any = None) -> Tuple[Any, Any, Any]:
-        """Run ``work`` with the communication stream current, ordered after the
-        inputs' producer and all consumers; returns (its value, the completion
-        event, the caller's stream)."""
+    def submit(self, work: Callable[[], Any], previous_event: Any = None, make_current: bool = True) -> Tuple[Any, Any, Any]:
+        """Put ``work`` on the communication stream, ordered after the inputs'
+        producer and all consumers; returns (its value, the completion event, the
+        caller's stream).  ``make_current`` makes the communication stream the
+        current one around ``work`` (needed by work that launches through PyTorch,
+        such as a graph replay); work that takes the stream explicitly skips that
+        switch, which is a measurable part of a small dispatch's CPU cost."""
         caller = torch.cuda.current_stream(self.device)
-        with torch.cuda.stream(self.stream):
-            ordered = {self._key(self.stream)}
-            if previous_event is None:
+        own_key = self._stream_key
+        if previous_event is None:
+            caller_key = (caller.device.index, int(caller.cuda_stream))
+            # A producer stream with nothing pending has produced the inputs already:
+            # asking is much cheaper than an event record plus a cross-stream wait.
+            if caller_key != own_key and not caller.query():
                 self.stream.wait_stream(caller)
-                ordered.add(self._key(caller))
-            elif isinstance(previous_event, EventOverlap):
-                previous_event.current_stream_wait()
+        else:
+            caller_key = own_key
+            if isinstance(previous_event, EventOverlap):
+                previous_event.stream_wait(self.stream)
             else:
                 self.stream.wait_event(previous_event)
+        if self._consumers:
             with self._guard:
                 consumers = list(self._consumers.items())
             for key, stream in consumers:
-                if key not in ordered:
+                if key != own_key and key != caller_key:
                     self.stream.wait_stream(stream)
+        if make_current:
+            with torch.cuda.stream(self.stream):
+                value = work()
+        else:
             value = work()
-            done = torch.cuda.Event()
-            done.record(self.stream)
+        done = torch.cuda.Event()
+        done.record(self.stream)
         return value, done, caller
 
 
@@ -212,9 +226,10 @@ class HostStagedEPBuffer:
 
     # ---- one admitted request -> outputs --------------------------------------------------
     def _launch(self, request: DispatchRequest, work: Callable[[], Dict[str, Any]], keep: tuple, previous_event: Any,
-                asynchronous: bool, deferred: bool = False) -> Any:
+                asynchronous: bool, deferred: bool = False, through_torch: bool = True) -> Any:
         """Put ``work`` (which returns the result dict) on the communication stream
-        and wrap the outcome.  ``keep`` is kept alive until the event is released."""
+        and wrap the outcome.  ``keep`` is kept alive until the event is released.
+        ``through_torch`` is false for work that is given the stream explicitly."""
         def on_comm_stream() -> Dict[str, Any]:
             record_tensors(request.inputs, self._ordering.stream)
             result = work()
@@ -223,7 +238,7 @@ class HostStagedEPBuffer:
                 request.stats_out.record_stream(self._ordering.stream)
             return result
 
-        result, done, caller = self._ordering.submit(on_comm_stream, previous_event)
+        result, done, caller = self._ordering.submit(on_comm_stream, previous_event, through_torch or request.stats_out is not None)
         overlap = EventOverlap(done, (self, request.inputs, request.stats_out, request.cached, result) + keep, self._ordering.saw_consumer)
         handle = HostStagedEPHandle(self, request.routes, result, request.expand, request.alignment, overlap)
         self._last_handle = handle
@@ -231,7 +246,11 @@ class HostStagedEPBuffer:
                    result.get("recv_topk_weights") if request.weights is not None else None, handle)
         if not asynchronous:
             caller.wait_event(done)
-            record_tensors(result, caller)
+            # The result tensors belong to a pool that was allocated on one stream
+            # and lives as long as the buffer; only a consumer on another stream
+            # needs to be made known to the caching allocator.
+            if self._ordering._key(caller) != self.runtime.allocation_stream:
+                record_tensors(result, caller)
             self._ordering.saw_consumer(caller)
         if deferred:
             overlap.register_hook_after_wait(lambda: outputs)
@@ -295,9 +314,9 @@ class HostStagedEPBuffer:
 
             def eager() -> Dict[str, Any]:
                 return self.runtime.dispatch(request.x, request.routes, request.weights, self.config.stage, request.alignment,
-                                             request.expand, request.zero_padding, request.plan, False)
+                                             request.expand, request.zero_padding, request.plan, False, stream=self._ordering.raw_stream)
 
-            return self._launch(request, eager, (), previous_event, async_with_compute_stream, defer_epilogue)
+            return self._launch(request, eager, (), previous_event, async_with_compute_stream, defer_epilogue, through_torch=False)
 
     def capture_dispatch(self, *args: Any, **kwargs: Any) -> Any:
         """Prepare the buffer's one fixed-address ``GraphDispatch`` (may synchronise)."""

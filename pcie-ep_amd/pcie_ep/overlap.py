@@ -64,6 +64,12 @@ class EventOverlap:
         self.event = self.extra_tensors = self._consumer_seen = None
 
     # ---- public forms -------------------------------------------------------------------
+    def stream_wait(self, stream: Any) -> Any:
+        """Order ``stream`` (rather than the current stream) after the event."""
+        if self.event is None:
+            raise RuntimeError("The event has already been released")
+        return self._attach(stream)
+
     def current_stream_wait(self, release_handle: bool = False) -> Any:
         if self.event is None:
             raise RuntimeError("The event has already been released")

@@ -56,13 +56,13 @@ class _Pool:
         }
         self._members = list(self.tensors.values())
         self._storages = [tensor.untyped_storage() for tensor in self._members]
+        self._storage_handles = [storage._cdata for storage in self._storages]  # the storages above keep them valid
         # Output pointers never change: the argument block is filled in once.
         self.arguments = _native.DispatchArgs(**{name: tensor.data_ptr() for name, tensor in self.tensors.items()})
         self._idle = self.references()
 
     def references(self) -> list:
-        use_count = torch._C._storage_Use_Count
-        return [sys.getrefcount(tensor) for tensor in self._members] + [use_count(storage._cdata) for storage in self._storages]
+        return list(map(sys.getrefcount, self._members)) + list(map(torch._C._storage_Use_Count, self._storage_handles))
 
     def idle(self) -> bool:
         return self.references() == self._idle
@@ -121,6 +121,8 @@ class NativeRuntime:
 
     # ---- allocation -----------------------------------------------------------------
     def _allocate(self) -> None:
+        allocating = torch.cuda.current_stream(self.device)
+        self.allocation_stream = (allocating.device.index, int(allocating.cuda_stream))
         n, capacity = int(self.sizes.unique_rows), int(self.sizes.expanded_rows)
         h, k, p, local, c = self.hidden, self.topk, self.world, int(self.sizes.local_experts), self.channels
         shapes = {
@@ -142,6 +144,7 @@ class NativeRuntime:
         self._plans: List[RoutePlan] = [RoutePlan(self.owner_id, int(self.sizes.plan_bytes), self.device) for _ in range(eager)]
         self._graph_plan = RoutePlan(self.owner_id, int(self.sizes.plan_bytes), self.device) if self.config.enable_graph else None
         self._plan_idle = self._plan_references(0)
+        self._last_pool = eager - 1
 
     def _plan_references(self, index: int) -> int:
         return sys.getrefcount(self._plans[index])
@@ -152,9 +155,14 @@ class NativeRuntime:
             if not self.config.enable_graph:
                 raise RuntimeError("Graph output pool was not prepared")
             return self._pools[self.config.output_pool_size]
-        for pool in self._pools[: self.config.output_pool_size]:
-            if pool.idle():
-                return pool
+        # Start after the pool used last: in a steady loop that one is still held
+        # by the caller and the next one has just been released.
+        eager = self.config.output_pool_size
+        for step in range(1, eager + 1):
+            index = (self._last_pool + step) % eager
+            if self._pools[index].idle():
+                self._last_pool = index
+                return self._pools[index]
         raise RuntimeError("preallocated output pool exhausted; release prior results or use a separate buffer")
 
     def _select_plan(self, tokens: int, cached_layout: Optional[RoutePlan], graph_pool: bool) -> RoutePlan:
@@ -173,9 +181,11 @@ class NativeRuntime:
         raise RuntimeError("preallocated route plan pool exhausted; release old handles/cache plans")
 
     def dispatch(self, x: torch.Tensor, idx: torch.Tensor, weights: Optional[torch.Tensor], stage: int, alignment: int,
-                 expand: bool, zero_padding: bool, cached_layout: Any = None, graph_pool: bool = False) -> Dict[str, Any]:
-        """Enqueue one dispatch on the current stream and return the result dict
-        (counterpart of ``AdvancedRuntime.dispatch``: advanced.hpp:126-156)."""
+                 expand: bool, zero_padding: bool, cached_layout: Any = None, graph_pool: bool = False,
+                 stream: Optional[int] = None) -> Dict[str, Any]:
+        """Enqueue one dispatch on ``stream`` (a raw stream handle; default: the
+        current stream) and return the result dict (counterpart of
+        ``AdvancedRuntime.dispatch``: advanced.hpp:126-156)."""
         if self._handle is None:
             raise RuntimeError("advanced runtime is closed or closing")
         if stage != self.config.stage:
@@ -191,7 +201,8 @@ class NativeRuntime:
         arguments.expand, arguments.zero_padding = int(expand), int(zero_padding)
         arguments.reuse_plan, arguments.plan = int(cached_layout is not None), plan.storage.data_ptr()
         arguments.expanded_capacity_rows = int(self.sizes.expanded_rows)
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
         entry = self._lib.pcie_ep_dispatch_static_scratch if self.use_static_scratch else self._lib.pcie_ep_dispatch
         _native.check(entry(self._handle, C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
         t = pool.tensors
