@@ -215,6 +215,16 @@ __device__ __forceinline__ void host_field_store(T* address, T value) {
     __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// One 16-byte load from host memory at a per-lane address with the system-scope
+// policy, complete on return.  Lanes that read neighbouring entries of a packed
+// queue are served by one request per line; a buffer load would need one
+// instruction per distinct queue base.
+__device__ __forceinline__ u32x4 host_load_b128_at(const void* address) {
+    u32x4 value;
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(value) : "v"(address) : "memory");
+    return value;
+}
+
 __device__ __forceinline__ void wait_memory_ops() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void compiler_barrier() { asm volatile("" ::: "memory"); }
 

@@ -440,7 +440,7 @@ bool PeerEmulator::source_progress(int rank, uint64_t epoch, bool& done, bool& q
         size_t kept = 0;
         for (int slot_index : state.pending_slots) {
             const uint64_t expected = state.pending_sequence[slot_index];
-            if (expected && acquire(signal_at(own, z_.ack_offset, size_t(slot_index) * z_.endpoints + endpoint)) != expected) {
+            if (expected && acquire(ack_at(z_, own, slot_index / z_.dims.payload_slots, slot_index % z_.dims.payload_slots, endpoint)) != expected) {
                 state.pending_slots[kept++] = slot_index;
             } else {
                 state.pending_sequence[slot_index] = 0;

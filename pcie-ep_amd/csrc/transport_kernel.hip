@@ -322,26 +322,40 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     // later dispatch may overwrite the mailbox (advanced_dispatch.cuh:213-225).
     bool relays_drained = z.dims.domains == 0;
     int drain_ordinal = produced > slots ? produced - slots : 0;
+    uint64_t next_drain_poll = 0;
     bool workers_finished = false;
     while (true) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
         if (workers_finished && !drained) {
-            // Each pass checks up to 64 / endpoints ordinals with one lane per endpoint.
-            const int per_pass = kWave / endpoints;
-            const int my_ordinal = drain_ordinal + lane / endpoints;
-            const int endpoint = lane % endpoints;
-            bool acked = true;
-            if (lane < per_pass * endpoints && my_ordinal < produced) {
-                const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
-                const uint32_t remote = endpoint_mask_of(z.dims, me, state.plan_mask[token]);
-                if ((remote >> endpoint) & 1u)
-                    acked = host_load(ack_at(z, own, channel, my_ordinal % slots, endpoint)) == sequence(epoch, token);
+            // Each pass checks up to 64 / endpoints ordinals of every endpoint; lanes of
+            // one endpoint read consecutive ACK words (one 64-byte read per eight slots).
+            // While the channel's receive side is still busy the drain is not what the
+            // kernel waits for: it then polls sparingly, so that the small reads do not
+            // compete with the row reads for the link.
+            if (broadcast_first(now_ticks() >= next_drain_poll ? 1 : 0)) {
+                const int per_pass = kWave / endpoints;
+                const int my_ordinal = drain_ordinal + lane % per_pass;
+                const int endpoint = lane / per_pass;
+                int missing_ordinal = 0x7FFFFFFF;
+                if (endpoint < endpoints && my_ordinal < produced) {
+                    const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
+                    const uint32_t remote = endpoint_mask_of(z.dims, me, state.plan_mask[token]);
+                    if (((remote >> endpoint) & 1u) && host_load(ack_at(z, own, channel, my_ordinal % slots, endpoint)) != sequence(epoch, token))
+                        missing_ordinal = my_ordinal;
+                }
+                for (int offset = 32; offset > 0; offset >>= 1) {
+                    const int other = __shfl_xor(missing_ordinal, offset);
+                    missing_ordinal = other < missing_ordinal ? other : missing_ordinal;
+                }
+                // Everything before the first miss is done.
+                drain_ordinal = missing_ordinal < drain_ordinal + per_pass ? missing_ordinal : drain_ordinal + per_pass;
+                if (drain_ordinal >= produced) drained = true;
+                else if (missing_ordinal != 0x7FFFFFFF) {
+                    const bool receive_busy = broadcast_first(int(device_load(&q.rx_finished[channel].value))) == 0;
+                    next_drain_poll = now_ticks() + (receive_busy ? 20 : 1) * state.clock_khz / 1000;
+                }
             }
-            const uint64_t missing = __ballot(!acked);
-            if (!missing) drain_ordinal += per_pass;
-            else drain_ordinal += __builtin_ctzll(missing) / endpoints;  // everything before the first miss is done
-            if (drain_ordinal >= produced) drained = true;
         }
         if (workers_finished && drained && !relays_drained) {
             bool done = true;
@@ -414,7 +428,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                                          : descriptor_at(z, segment, channel, me, want ? ordinal : 0);
         // One 16-byte load brings READY together with the slot and token it guards.
         u32x4 published = {0u, 0u, 0u, 0u};
-        if (want) published = host_load_b128(host_resource(descriptor, 16), 0);
+        if (want) published = host_load_b128_at(descriptor);
         const bool ready = want && (uint64_t(published[0]) | uint64_t(published[1]) << 32) == sequence(epoch, ordinal);
         const uint64_t ready_lanes = __ballot(ready);
         // Descriptors of one source are consumed in order: accept the leading run.
@@ -709,8 +723,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
             atomicAdd(reinterpret_cast<unsigned long long*>(state.receive_expand_overlap + channel * 2), 1ull);
 
         // Metadata first (it arrives first), payload right behind it.
-        const uint32_t meta_lo = host_load_b32(slot_meta, uint32_t(lane) * 4u);  // out of range reads as 0
-        const uint32_t meta_hi = host_load_b32(slot_meta, uint32_t(kWave + lane) * 4u);
+        const u32x4 meta_vector = host_load_b128(slot_meta, uint32_t(lane) * 16u);  // 16 bytes per lane; out of range reads as 0
 
         RowVectors row;
         const int wire_vectors = kFp8 ? hidden / 16 : hidden / 8;
@@ -725,8 +738,12 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
                 for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(j * kWave + lane) * 16u);
             }
         }
-        scratch[lane] = meta_lo;
-        scratch[kWave + lane] = meta_hi;
+        if (lane < kScratchDwords / 4) {
+            scratch[lane * 4] = meta_vector[0];
+            scratch[lane * 4 + 1] = meta_vector[1];
+            scratch[lane * 4 + 2] = meta_vector[2];
+            scratch[lane * 4 + 3] = meta_vector[3];
+        }
         fence_lds();
         const int token = int(scratch[0]);
         const float scale = bits_float(scratch[2]);

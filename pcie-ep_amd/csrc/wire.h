@@ -4,7 +4,7 @@
 // One *segment* of pinned, fine-grained host memory exists per source rank.
 // Only the source writes payload slots, slot metadata, descriptor bodies,
 // READY words, the count mailbox, counts_ready, abort and channel_abort; a
-// receiver d writes only ack[..][d], the credit word of its own (s -> d)
+// receiver d writes only its ack[channel][d][..] array, the credit word of its own (s -> d)
 // descriptor queue and counts_consumed[d].  Every 64-bit signal therefore has
 // exactly one writer and nothing ever performs a read-modify-write on host
 // memory (the discipline of the reference: csrc/kernels/host_staged/common.cuh:59-64).
@@ -159,7 +159,8 @@ struct SegmentLayout {
     size_t channel_abort_offset;    // [C] signals
     size_t mailbox_offset;          // [P] blocks
     size_t slots_offset;            // [C*Q] slots, page aligned
-    size_t ack_offset;              // [C*Q][P] signals
+    size_t ack_offset;              // [C][P+N] arrays of Q words, one array (one writer) per 128-byte aligned block
+    size_t ack_stride;              // bytes of one such array
     size_t descriptors_offset;      // [C][P] queues of L packed entries, each queue 128-byte aligned
     size_t descriptor_queue_stride;
     size_t credits_offset;          // [C][P+N] signals: sequence(epoch, last ordinal the destination consumed)
@@ -167,7 +168,8 @@ struct SegmentLayout {
     int endpoints;                  // P + N
     size_t relay_mailbox_offset;    // [N] blocks of C dwords: tokens of each channel bound for the domain through the relay
     size_t relay_mailbox_stride;
-    size_t replica_ack_offset;      // [C][N][R][P] signals
+    size_t replica_ack_offset;      // [C][N][P] arrays of R words
+    size_t replica_ack_stride;
     size_t replica_descriptors_offset;  // [C][N][P] queues of L packed entries
     size_t replica_credits_offset;  // [C][N][P] signals
     size_t relay_drained_offset;    // [C][N] signals: epoch whose flow has been copied and released
@@ -208,12 +210,17 @@ PCIE_EP_HD SegmentLayout make_segment_layout(const Dimensions& dims) {
     cursor = align_up(cursor, kPageBytes);
     const size_t slots = size_t(dims.channels) * dims.payload_slots;
     z.slots_offset = reserve(slots * z.slot_stride);
-    z.ack_offset = reserve(slots * z.endpoints * sizeof(Signal));
+    // Payload ACKs: receiver d owns the array [channel][d] and stores sequence(epoch, token) into word
+    // `slot` once it has read that slot.  Grouped by writer, a line still has one writer, and the source's
+    // drain reads eight consecutive slots of one receiver with a single 64-byte read.
+    z.ack_stride = align_up(size_t(dims.payload_slots) * 8, kSignalBytes);
+    z.ack_offset = reserve(size_t(dims.channels) * z.endpoints * z.ack_stride);
     z.descriptor_queue_stride = align_up(size_t(dims.descriptor_slots) * sizeof(Descriptor), kSignalBytes);
     z.descriptors_offset = reserve(size_t(dims.channels) * z.endpoints * z.descriptor_queue_stride);
     z.credits_offset = reserve(size_t(dims.channels) * z.endpoints * sizeof(Signal));
     const size_t flows = size_t(dims.channels) * dims.domains;
-    z.replica_ack_offset = reserve(flows * dims.replica_slots * dims.num_ranks * sizeof(Signal));
+    z.replica_ack_stride = align_up(size_t(dims.replica_slots) * 8, kSignalBytes);
+    z.replica_ack_offset = reserve(flows * dims.num_ranks * z.replica_ack_stride);
     z.replica_descriptors_offset = reserve(flows * dims.num_ranks * z.descriptor_queue_stride);
     z.replica_credits_offset = reserve(flows * dims.num_ranks * sizeof(Signal));
     z.relay_drained_offset = reserve(flows * sizeof(Signal));
@@ -252,7 +259,7 @@ PCIE_EP_HD char* slot_at(const SegmentLayout& z, char* segment, int channel, int
 }
 // `endpoint` is a destination rank or, in relay mode, P + domain.
 PCIE_EP_HD uint64_t* ack_at(const SegmentLayout& z, char* segment, int channel, int slot, int endpoint) {
-    return signal_at(segment, z.ack_offset, (size_t(channel) * z.dims.payload_slots + slot) * z.endpoints + endpoint);
+    return reinterpret_cast<uint64_t*>(segment + z.ack_offset + (size_t(channel) * z.endpoints + endpoint) * z.ack_stride) + slot;
 }
 PCIE_EP_HD Descriptor* descriptor_at(const SegmentLayout& z, char* segment, int channel, int endpoint, int ordinal) {
     char* queue = segment + z.descriptors_offset + (size_t(channel) * z.endpoints + endpoint) * z.descriptor_queue_stride;
@@ -268,7 +275,7 @@ PCIE_EP_HD char* replica_slot_at(const SegmentLayout& z, char* region, int chann
     return region + (size_t(channel) * z.dims.replica_slots + slot) * z.slot_stride;
 }
 PCIE_EP_HD uint64_t* replica_ack_at(const SegmentLayout& z, char* segment, int channel, int domain, int slot, int destination) {
-    return signal_at(segment, z.replica_ack_offset, (flow_index(z, channel, domain) * z.dims.replica_slots + slot) * z.dims.num_ranks + destination);
+    return reinterpret_cast<uint64_t*>(segment + z.replica_ack_offset + (flow_index(z, channel, domain) * z.dims.num_ranks + destination) * z.replica_ack_stride) + slot;
 }
 PCIE_EP_HD Descriptor* replica_descriptor_at(const SegmentLayout& z, char* segment, int channel, int domain, int destination, int ordinal) {
     char* queue = segment + z.replica_descriptors_offset + (flow_index(z, channel, domain) * z.dims.num_ranks + destination) * z.descriptor_queue_stride;
