@@ -18,7 +18,14 @@ constexpr int kDefaultTxWaves = 2;
 constexpr int kDefaultRxWaves = 2;
 constexpr int kMaxTxWaves = 4;
 constexpr int kMaxRxWaves = 6;
-constexpr int kMaxWorkerGroups = 1024;
+// Upper bound of the payload workgroups: with at most 32 control and 32 local-bypass workgroups the grid then has at
+// most 256 workgroups of at most 768 threads, and an MI355X (256 compute units, each able to hold at least one such
+// workgroup next to other work) keeps all of them resident at once.  The roles wait for each other through device
+// memory, so the control workgroups must be running while payload wavefronts wait for tickets: with the whole grid
+// resident that holds without any assumption about the order in which workgroups are started.  On a smaller
+// partition the control workgroups still carry the lowest indices and are started first; should a payload wavefront
+// ever wait for a control workgroup that is not running, its bounded wait ends the dispatch with code 15.
+constexpr int kMaxWorkerGroups = 192;
 
 // Workgroup sizes.  Each constant is used twice: as the __launch_bounds__ of the
 // kernel and by its launcher, so a launch shape can never exceed what the kernel

@@ -38,6 +38,7 @@ from .overlap import EventOverlap, record_tensors
 from .peers import PeerGroup
 from .request import DispatchRequest, admit
 from .runtime import NativeRuntime
+from .streams import MaskedStream
 
 _next_buffer_id = itertools.count(1)
 
@@ -45,9 +46,11 @@ _next_buffer_id = itertools.count(1)
 class _Ordering:
     """Stream ordering of one buffer."""
 
-    def __init__(self, device: int) -> None:
+    def __init__(self, device: int, compute_units: int = 0) -> None:
         self.device = device
-        self.stream = torch.cuda.Stream(device=device)
+        # Optionally confine the dispatch kernels to the first `compute_units` units.
+        self.masked = MaskedStream(device, compute_units) if compute_units else None
+        self.stream = self.masked.stream if self.masked else torch.cuda.Stream(device=device)
         self.stream.wait_stream(torch.cuda.current_stream(device))
         self._stream_key = self._key(self.stream)
         self.raw_stream = int(self.stream.cuda_stream)
@@ -70,6 +73,9 @@ class _Ordering:
     def forget(self) -> None:
         with self._guard:
             self._consumers.clear()
+        if self.masked is not None:
+            self.masked.close()
+            self.masked = None
 
     def submit(self, work: Callable[[], Any], previous_event: Any = None, make_current: bool = True) -> Tuple[Any, Any, Any]:
         """Put ``work`` on the communication stream, ordered after the inputs'
@@ -132,6 +138,7 @@ class HostStagedEPBuffer:
         rx_waves: int = 0,
         worker_groups: int = 0,
         rank_numa_nodes: Optional[Tuple[int, ...]] = None,
+        comm_stream_cus: int = 0,
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
@@ -150,6 +157,10 @@ class HostStagedEPBuffer:
         which the reference gathers from its processes; ranks of another node than
         a source's are reached through that source's relay workers and replica
         rings.  Default: every rank on the GPU's node, i.e. one domain.
+        ``comm_stream_cus`` > 0 confines the dispatch kernels to that many compute
+        units (``pcie_ep.streams``), so that compute kernels on a stream masked to
+        the remaining units run undisturbed while a dispatch is in flight; 64 units
+        carry the dispatch at full link rate.
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -186,7 +197,7 @@ class HostStagedEPBuffer:
         self._state = "live"  # "live" -> "failed" | "closed"
         self._last_handle: Optional[HostStagedEPHandle] = None
         self._graph_capture = None
-        self._ordering = _Ordering(self.device)
+        self._ordering = _Ordering(self.device, comm_stream_cus)
         self.runtime: Optional[NativeRuntime] = None
         threads = min(num_ranks - 1, 7) if peer_threads is None else peer_threads
         if rank_numa_nodes is not None:

@@ -230,6 +230,50 @@ def test_dispatch_overlaps_with_compute_on_another_stream():
             del result
 
 
+def test_dispatch_confined_to_a_subset_of_the_compute_units():
+    """``comm_stream_cus``: the dispatch kernels run on a stream masked to 64
+    compute units while GEMMs run on a stream masked to the other 192; results,
+    cached layouts and graph replays are unchanged."""
+    from helpers import baseline_inputs
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+    from pcie_ep.streams import masked_stream
+
+    tokens = 1024
+    inputs = baseline_inputs(tokens, 8)
+    total = torch.cuda.get_device_properties(0).multi_processor_count
+    with pytest.raises(ValueError, match="does not fit"):
+        masked_stream(total + 1)
+    compute = masked_stream(total - 64, first=64)
+    with HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=7168, num_topk=8, num_experts=256,
+                            config=HostStagedConfig(channels=32, timeout_ms=20_000, enable_graph=True), num_ranks=8, rank=0,
+                            comm_stream_cus=64) as buffer:
+        assert buffer.get_comm_stream().cuda_stream == buffer._ordering.masked.stream.cuda_stream
+        x, idx, weights = (item.cuda() for item in inputs[0])
+        a = torch.randn(4096, 4096, device="cuda", dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        print("case: masked communication stream (64 CUs) with GEMMs on the other compute units", flush=True)
+        arm(buffer, inputs)
+        with torch.cuda.stream(compute.stream):
+            c = a
+            for _ in range(30):
+                c = (a @ c).clamp_(-1, 1)
+        result = buffer.dispatch(x, idx, weights, do_expand=True)
+        verify_dispatch(result, inputs, 0, WORLD, 256, 8, True, 1, False)
+        buffer.peers.wait(30_000)
+        cache = buffer.cache_layout(result[3])
+        del result
+        graph = buffer.capture_dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
+        for _ in range(2):
+            arm(buffer, inputs)
+            replayed = graph.replay()
+            verify_dispatch(replayed, inputs, 0, WORLD, 256, 8, True, 1, False)
+            buffer.peers.wait(30_000)
+            del replayed
+        compute.stream.synchronize()
+        assert torch.isfinite(c.float().sum())
+    compute.close()
+
+
 def test_misaligned_payload_is_refused_by_the_native_boundary(inputs):
     """Rows move as 16-byte vectors: a contiguous tensor whose storage offset breaks
     that alignment must be rejected on the host, never handed to a kernel."""

@@ -107,7 +107,7 @@ def test_large_hidden_multi_pass():
 
 
 def test_wave_counts():
-    for tx_waves, rx_waves, helpers in ((1, 1, -1), (4, 6, 3), (2, 2, 300)):
+    for tx_waves, rx_waves, helpers in ((1, 1, -1), (4, 6, 3), (2, 2, 192)):
         with make_buffer(hidden=512, channels=4, payload_slots=2, descriptor_slots=2, tx_waves=tx_waves, rx_waves=rx_waves,
                          worker_groups=helpers) as buffer:
             check_case(buffer, f"tx{tx_waves}rx{rx_waves}h{helpers}", [60] * 8)
