@@ -187,7 +187,7 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
 
         ceilings = {}
         extra = max(0, min(1024, round((expanded / max(unique, 1) - 1.0) * 1024)))
-        for name, pattern in (("linear", 0), ("expert_streams", 1), ("hashed", 2)):
+        for name, pattern in (("linear", 0), ("expert_streams", 1), ("hashed", 2), ("read_only", 3), ("write_only", 4)):
             rate = _native.C.c_double()
             _native.check(_native.library().pcie_ep_measure_row_scatter(0, unique, HIDDEN * 2, extra, pattern, EXPERTS // WORLD, 5, _native.C.byref(rate)),
                           invalid=RuntimeError)

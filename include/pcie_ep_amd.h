@@ -289,7 +289,8 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
  * without its metadata: every wavefront reads one row of `row_bytes` and writes
  * it once, `extra_per_1024` of every 1024 rows twice.  pattern 0 writes in linear
  * order, 1 into `streams` interleaved sequential streams (what expert-major
- * placement of source-ordered rows produces), 2 hashed.  The practical HBM
+ * placement of source-ordered rows produces), 2 hashed, 3 reads the rows only,
+ * 4 writes them only (one row per wavefront each).  The practical HBM
  * ceiling for a write-heavy row scatter on this part.  No counterpart in the
  * reference. */
 int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes, int32_t extra_per_1024, int32_t pattern, int32_t streams,

@@ -50,7 +50,7 @@ hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
 // Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.
 hipError_t launch_copy(const void* source, void* destination, int64_t bytes, hipStream_t stream);
 // One row read, one row written (and `extra_per_1024` of every 1024 rows written a second time into the upper half of
-// `destination`, which holds 2 * rows rows): pattern 0 linear, 1 `streams` interleaved sequential streams, 2 hashed.
+// `destination`, which holds 2 * rows rows): pattern 0 linear, 1 `streams` interleaved sequential streams, 2 hashed, 3 read only, 4 write only.
 hipError_t launch_row_scatter(const void* source, void* destination, int rows, int row_bytes, int extra_per_1024, int pattern, int streams,
                               hipStream_t stream);
 // Zero `bytes` (a multiple of 16) of device memory at a 16-byte aligned address with a fill kernel.

@@ -858,7 +858,7 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
 
 int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes, int32_t extra_per_1024, int32_t pattern, int32_t streams,
                                 int32_t repeats, double* gbps) {
-    if (rows < 1 || row_bytes < 16 || row_bytes % 16 || extra_per_1024 < 0 || extra_per_1024 > 1024 || pattern < 0 || pattern > 2 || streams < 1 ||
+    if (rows < 1 || row_bytes < 16 || row_bytes % 16 || extra_per_1024 < 0 || extra_per_1024 > 1024 || pattern < 0 || pattern > 4 || streams < 1 ||
         repeats < 1 || !gbps)
         return set_error(PCIE_EP_E_INVALID, "bad measurement arguments");
     HIP_TRY(hipSetDevice(device));
@@ -884,7 +884,9 @@ int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes,
         float ms = 0.0f;
         if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
         if (status == hipSuccess && i > 0 && ms > 0.0f) {
-            const double rate = double(2 * int64_t(rows) + twice) * double(row_bytes) / (ms * 1e6);  // bytes read + bytes written
+            // bytes read + bytes written; the read-only and write-only patterns move every row once
+            const double moved = pattern >= 3 ? double(rows) : double(2 * int64_t(rows) + twice);
+            const double rate = moved * double(row_bytes) / (ms * 1e6);
             if (rate > best) best = rate;
         }
     }
