@@ -31,6 +31,13 @@
 //    every control-path read, from the number of channels.
 //  * Workers publish their own descriptors and payload ACKs as soon as their own
 //    stores / loads have completed; control wavefronts only reserve and hand out.
+//  * A payload wavefront has a home direction (transmit or receive) but is not
+//    bound to it: once every ticket of its own direction has been claimed it
+//    takes tickets of the other one, so both directions end together whatever
+//    the routing's send/receive ratio is.
+//  * Every read from host memory is a whole 16-byte vector per lane (payload, slot
+//    metadata, descriptor entries) or a packed word array (ACKs): small scattered
+//    reads cost the host link far more than their bytes.
 //  * The workgroups after the payload workgroups do the local bypass (own tokens
 //    routed to own experts: advanced_copy_local_tokens, advanced_layout.cuh:217-248)
 //    and the zeroing of the alignment gaps (:250-265) as soon as the receive
@@ -943,7 +950,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
                 const bool tx_done = tx_total >= 0 && tx_head >= tx_total, rx_done = rx_total >= 0 && rx_head >= rx_total;
                 if (home_tx ? tx_backlog : rx_backlog) choice = home_tx ? 1 : 2;
                 else if ((home_tx ? tx_done : rx_done) && (home_tx ? rx_backlog : tx_backlog)) choice = home_tx ? 2 : 1;
-                else {
+                if (choice == 0) {
                     if (tx_done && rx_done) choice = -1;
                     else if (deadline.expired(state)) {
                         record_error(state, kErrRingProgressWait);
