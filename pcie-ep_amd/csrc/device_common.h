@@ -11,6 +11,9 @@ namespace pcie_ep {
 
 constexpr int kWave = 64;
 constexpr uint64_t kPrefixFailed = ~uint64_t(0);
+// Set in the claim word of the receive prefixes once their producer has put its
+// reads of the count mailboxes on the host link.
+constexpr uint64_t kPrefixRequested = uint64_t(1) << 63;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

@@ -129,10 +129,16 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         state.prefix_tx_timestamps_ns[0] = ticks_to_ns(state, start);
         test_delay(state.prefix_delay);
     }
+    // This runs while the payload wavefronts already stream rows, so it keeps to
+    // the discipline of the hot path: host words are read with the system-scope
+    // policy (never from a GPU cache, so no invalidate is needed), results are
+    // written through to device memory (so no cache write-back is needed), and
+    // ordering is by waiting for this wavefront's own operations.  A cache
+    // write-back here would have to flush the rows the scatter is writing.
     // All sources are polled in parallel, one lane each.
     bool ready = lane >= ranks;
     while (true) {
-        if (!ready) ready = load_acquire_system(signal_at(state.seg[lane], z.counts_ready_offset)) == epoch;
+        if (!ready) ready = host_load(signal_at(state.seg[lane], z.counts_ready_offset)) == epoch;
         if (__all(ready)) break;
         if (health.poll(state, lane)) {
             if (lane == 0) record_error(state, kErrCountsReadyWait);
@@ -140,17 +146,34 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         }
         backoff();
     }
-    fence_acquire_system();
-    // Per-source unique counts -> source_offsets (lane = source).
+    // Every mailbox word this wavefront needs is requested now, before the first
+    // one is used: one round trip over the host link instead of one per group.
     int unique = 0;
-    if (lane < ranks) unique = mailbox_at(z, state.seg[lane], me)[0];
+    if (lane < ranks) unique = host_field_load(mailbox_at(z, state.seg[lane], me));
+    constexpr int kExpectedPerLane = kMaxChannels * kMaxRanks / kWave;
+    int expected_values[kExpectedPerLane];
+#pragma unroll
+    for (int i = 0; i < kExpectedPerLane; ++i) {
+        const int index = lane + i * kWave;
+        expected_values[i] = index < channels * ranks ? host_field_load(mailbox_at(z, state.seg[index % ranks], me) + 1 + local + index / ranks) : 0;
+    }
+    int first_counts[kMaxRanks];
+#pragma unroll
+    for (int source = 0; source < kMaxRanks; ++source)
+        first_counts[source] = (source < ranks && lane < local) ? host_field_load(mailbox_at(z, state.seg[source], me) + 1 + lane) : 0;
+    // The reads are on the link (requests leave in issue order): the receive side
+    // may now flood it with row reads without delaying these few words.
+    compiler_barrier();
+    if (lane == 0) device_store(state.receive_prefix_state, epoch | kPrefixRequested);
+    compiler_barrier();
+    // Per-source unique counts -> source_offsets (lane = source).
     int inclusive = unique;
     for (int offset = 1; offset < kMaxRanks; offset <<= 1) {
         const int other = __shfl_up(inclusive, offset);
         if (lane >= offset) inclusive += other;
     }
-    if (lane < ranks) state.source_offsets[lane + 1] = inclusive;
-    if (lane == 0) state.source_offsets[0] = 0;
+    if (lane < ranks) device_store(state.source_offsets + lane + 1, inclusive);
+    if (lane == 0) device_store(state.source_offsets, 0);
     const int total_unique = __shfl(inclusive, ranks - 1);
     // Expert branches: lane = local expert; all sources' loads are issued first.
     int carry_offset = 0;
@@ -159,12 +182,14 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         const int expert = begin + lane;
         int counts[kMaxRanks];
 #pragma unroll
-        for (int source = 0; source < kMaxRanks; ++source)
-            counts[source] = (source < ranks && expert < local) ? mailbox_at(z, state.seg[source], me)[1 + expert] : 0;
+        for (int source = 0; source < kMaxRanks; ++source) {
+            if (begin == 0) counts[source] = first_counts[source];
+            else counts[source] = (source < ranks && expert < local) ? host_field_load(mailbox_at(z, state.seg[source], me) + 1 + expert) : 0;
+        }
         int running = 0;
 #pragma unroll
         for (int source = 0; source < kMaxRanks; ++source) {
-            if (source < ranks && expert < local) state.source_expert_prefix[source * local + expert] = running;
+            if (source < ranks && expert < local) device_store(state.source_expert_prefix + source * local + expert, running);
             running += counts[source];
         }
         const int padded = (running + state.alignment - 1) / state.alignment * state.alignment;
@@ -175,10 +200,10 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         }
         const int exclusive = carry_offset + scan - padded;
         if (expert < local) {
-            state.expert_counts[expert] = running;
-            state.expert_offsets[expert] = exclusive;
-            state.expert_prefix[expert] = exclusive + running;
-            if (expert == local - 1) state.expert_offsets[local] = exclusive + padded;
+            device_store(state.expert_counts + expert, running);
+            device_store(state.expert_offsets + expert, exclusive);
+            device_store(state.expert_prefix + expert, exclusive + running);
+            if (expert == local - 1) device_store(state.expert_offsets + local, exclusive + padded);
         }
         carry_offset += __shfl(scan, kWave - 1);
         int sum = running;
@@ -186,53 +211,65 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         expanded_total += sum;
     }
     // Expected tokens per (channel, source) for this receiver.
-    for (int index = lane; index < channels * ranks; index += kWave) {
-        const int channel = index / ranks, source = index % ranks;
-        state.expected_receive_counts[index] = mailbox_at(z, state.seg[source], me)[1 + local + channel];
+#pragma unroll
+    for (int i = 0; i < kExpectedPerLane; ++i) {
+        const int index = lane + i * kWave;
+        if (index < channels * ranks) device_store(state.expected_receive_counts + index, expected_values[i]);
     }
     const int own_unique = __shfl(unique, me);
     if (lane == 0) {
-        *state.unique_count = total_unique;
-        *state.expanded_count = expanded_total;
+        device_store(state.unique_count, int64_t(total_unique));
+        device_store(state.expanded_count, expanded_total);
         // Receive tickets of this dispatch: every unique row of a remote source.
         device_store(&state.queues->rx_head.total, total_unique - own_unique);
     }
-    // ACK a source only after every lane captured its counts: the source may
-    // overwrite the mailbox for the next epoch afterwards (advanced_layout.cuh:91-93).
-    __threadfence_system();
-    if (lane < ranks && lane != me && lane != state.counts_ack_skip_source)
-        store_release_system(signal_at(state.seg[lane], z.counts_consumed_offset, me), epoch);
     return true;
 }
 
-__device__ bool prepare_receive_prefixes(const DeviceState& state, int lane) {
+// A source may overwrite its count mailbox for the next epoch once this rank has
+// said so.  Every lane has its counts in registers by now (the loads above were
+// waited for, wave-wide), so the ACK needs no fence (advanced_layout.cuh:91-93).
+__device__ void acknowledge_counts(const DeviceState& state, int lane) {
+    const SegmentLayout& z = state.z;
+    wait_memory_ops();
+    if (lane < z.dims.num_ranks && lane != state.local_rank && lane != state.counts_ack_skip_source)
+        host_field_store(signal_at(state.seg[lane], z.counts_consumed_offset, state.local_rank), *state.epoch);
+}
+
+// One wavefront of the grid (the first RX control to get there) computes the
+// receive prefixes; nobody waits here.
+__device__ void elect_receive_prefixes(const DeviceState& state, int lane) {
     const uint64_t epoch = *state.epoch;
     int claimed = 0;
     if (lane == 0) {
         unsigned long long expected = 0;
         claimed = atomicCAS(reinterpret_cast<unsigned long long*>(state.receive_prefix_state), expected, epoch) == 0ull;
     }
-    if (broadcast_first(claimed)) {
-        const bool success = compute_receive_prefixes(state, lane);
-        __threadfence();
-        if (lane == 0) {
-            state.prefix_tx_timestamps_ns[1] = ticks_to_ns(state, now_ticks());
-            store_release_device(state.receive_prefix_state + 1, success ? epoch : kPrefixFailed);
-        }
-    }
-    int success = 0;
+    if (!broadcast_first(claimed)) return;
+    const bool success = compute_receive_prefixes(state, lane);
+    // The results were written through; they are complete once this wavefront's
+    // stores have been acknowledged.  Local consumers come first, the ACK to the
+    // sources (which nobody on this GPU waits for) second.
+    wait_memory_ops();
     if (lane == 0) {
-        while (true) {
-            const uint64_t value = load_acquire_device(state.receive_prefix_state + 1);
-            if (value == epoch) { success = 1; break; }
-            // The elected producer owns the timeout; waiters only read device flags.
-            if (value == kPrefixFailed || load_error_code(state)) break;
-            backoff();
-        }
+        state.prefix_tx_timestamps_ns[1] = ticks_to_ns(state, now_ticks());
+        device_store(state.receive_prefix_state + 1, success ? epoch : kPrefixFailed);
     }
-    success = broadcast_first(success);
-    __threadfence();
-    return success != 0;
+    if (success) acknowledge_counts(state, lane);
+}
+
+// 1 once the receive prefixes of this epoch are published, -1 when they never
+// will be (their producer failed or the dispatch has an error), 0 otherwise.
+// The elected producer owns the timeout; everybody else only reads device flags.
+__device__ __forceinline__ int receive_prefix_verdict(const DeviceState& state, uint64_t epoch, int lane) {
+    int verdict = 0;
+    if (lane == 0) {
+        // Relaxed: what the flag guards is read with device-scope loads.
+        const uint64_t value = device_load(state.receive_prefix_state + 1);
+        if (value == epoch) verdict = 1;
+        else if (value == kPrefixFailed || load_error_code(state)) verdict = -1;
+    }
+    return broadcast_first(verdict);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -340,7 +377,8 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
             // While the channel's receive side is still busy the drain is not what the
             // kernel waits for: it then polls sparingly, so that the small reads do not
             // compete with the row reads for the link.
-            if (broadcast_first(now_ticks() >= next_drain_poll ? 1 : 0)) {
+            const bool receive_busy = broadcast_first(int(device_load(&q.rx_finished[channel].value))) == 0;
+            if (!receive_busy || broadcast_first(now_ticks() >= next_drain_poll ? 1 : 0)) {
                 const int per_pass = kWave / endpoints;
                 const int my_ordinal = drain_ordinal + lane % per_pass;
                 const int endpoint = lane / per_pass;
@@ -358,10 +396,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
                 // Everything before the first miss is done.
                 drain_ordinal = missing_ordinal < drain_ordinal + per_pass ? missing_ordinal : drain_ordinal + per_pass;
                 if (drain_ordinal >= produced) drained = true;
-                else if (missing_ordinal != 0x7FFFFFFF) {
-                    const bool receive_busy = broadcast_first(int(device_load(&q.rx_finished[channel].value))) == 0;
-                    next_drain_poll = now_ticks() + (receive_busy ? 20 : 1) * state.clock_khz / 1000;
-                }
+                else if (missing_ordinal != 0x7FFFFFFF) next_drain_poll = now_ticks() + 20 * state.clock_khz / 1000;
             }
         }
         if (workers_finished && drained && !relays_drained) {
@@ -401,22 +436,35 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, me = state.local_rank;
     const uint64_t begin = now_ticks();
-    if (!prepare_receive_prefixes(state, lane)) {
-        if (lane == 0) {
-            raise_abort(q);
-            device_store(&q.rx_finished[channel].value, 1u);
-        }
-        return;
-    }
     const uint64_t epoch = *state.epoch;
+    elect_receive_prefixes(state, lane);
+    // Polling does not wait for the prefixes: a descriptor entry is valid as soon as
+    // its tag carries this epoch and the next ordinal, whatever the counts say, so
+    // rows are requested from the first microseconds of the kernel on.  The counts
+    // (how many rows each source sends on this channel) are only needed to know
+    // when to stop; the payload wavefronts wait for the prefixes after they have
+    // requested a row, before they compute where it goes.
     const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
     const int source = lane / lookahead, ahead = lane % lookahead;
     const bool member = source < ranks && source != me;
     const bool replica = member && reads_replica(z.dims, source, me);
     const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
-    const int expected = member ? state.expected_receive_counts[channel * ranks + source] : 0;
-    int total = ahead == 0 ? expected : 0;
-    for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
+    int expected = member ? 0x7FFFFFFF : 0, total = 0x7FFFFFFF;
+    bool counts_known = false, prefix_failed = false;
+    // ... but not before the producer of the prefixes has requested the count
+    // mailboxes: a few hundred bytes that everything waits for must not queue
+    // behind megabytes of row reads.
+    while (true) {
+        int gate = 0;
+        if (lane == 0) gate = (device_load(state.receive_prefix_state) & kPrefixRequested) ? 1 : (aborted(q) ? -1 : 0);
+        gate = broadcast_first(gate);
+        if (gate > 0) break;
+        if (gate < 0 || receive_prefix_verdict(state, epoch, lane) < 0) {
+            prefix_failed = true;
+            break;
+        }
+        backoff();
+    }
     const uint64_t below = lanes_below(lane);
     const uint64_t group_mask = (1ull << lookahead) - 1ull;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
@@ -424,8 +472,22 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     int consumed = 0, issued = 0;
     int64_t not_ready = 0, ring_waits = 0;
     bool failed = false;
-    while (issued < total && !failed) {
+    while (!failed && !prefix_failed) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
+        if (!counts_known) {
+            const int verdict = receive_prefix_verdict(state, epoch, lane);
+            if (verdict < 0) {
+                prefix_failed = true;
+                break;
+            }
+            if (verdict > 0) {
+                expected = member ? device_load(state.expected_receive_counts + channel * ranks + source) : 0;
+                total = ahead == 0 ? expected : 0;
+                for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
+                counts_known = true;
+            }
+        }
+        if (counts_known && issued >= total) break;
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
         // A source of another domain is read from the replica ring its relay fills
@@ -485,6 +547,13 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                              sequence(epoch, consumed + run - 1));
         if (member) consumed += run;
     }
+    if (prefix_failed) {
+        if (lane == 0) {
+            raise_abort(q);
+            device_store(&q.rx_finished[channel].value, 1u);
+        }
+        return;
+    }
     // RX is finished when every ticket has been retired by a worker.
     while (true) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
@@ -516,7 +585,7 @@ __device__ void local_rows(const DeviceState& state, TransportQueues& q, int lan
     int ready = 0;
     if (lane == 0) {
         while (true) {
-            const uint64_t value = load_acquire_device(state.receive_prefix_state + 1);
+            const uint64_t value = device_load(state.receive_prefix_state + 1);  // what it guards is read with device-scope loads
             if (value == epoch) { ready = 1; break; }
             // The wavefront that computes the prefixes owns the timeout.
             if (value == kPrefixFailed || aborted(q) || load_error_code(state)) break;
@@ -697,7 +766,8 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 // host slot and stores it to its destination rows.  Returns false when the
 // wavefront must stop.
 template <bool kFp8, bool kVector>
-__device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters) {
+__device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters,
+                       bool& prefixes_known) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
@@ -762,6 +832,15 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
                 raise_abort(q);
             }
             return false;
+        }
+
+        // The row has been requested; where it goes depends on the receive prefixes,
+        // which may still be on their way in the first microseconds of the kernel.
+        while (!prefixes_known) {
+            const int verdict = receive_prefix_verdict(state, epoch, lane);
+            if (verdict < 0 || broadcast_first(aborted(q) ? 1 : 0)) return false;
+            if (verdict > 0) prefixes_known = true;
+            else backoff();
         }
 
         // Destination rows, one lane per branch.  Everything the row numbers are
@@ -937,6 +1016,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
     const uint64_t epoch = *state.epoch;
     Deadline deadline(now_ticks());
     WorkerCounters counters;
+    bool prefixes_known = false;
     while (true) {
         // 0: nothing to do now, 1: transmit, 2: receive, -1: both directions are finished or the kernel aborts.
         int choice = 0;
@@ -976,7 +1056,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
             continue;
         }
         const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters)
-                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters);
+                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, prefixes_known);
         if (!go_on) break;
     }
     // Workers serve every channel; their counts go to channel 0's row of the
