@@ -115,6 +115,44 @@ def test_relay_with_one_domain_carries_nothing():
         check_flows(buffer.runtime.relay_diagnostics(), 0, 2048)
 
 
+def test_relay_workers_are_pinned_to_the_requested_cpus():
+    """``relay_cpu_affinity`` restricts the CPUs the workers of an existing node are
+    pinned to (numa_relay.hpp:178-199); workers of a node this machine does not
+    have stay unpinned.  Cached layouts and graph replays work through the relay."""
+    import os
+
+    allowed = sorted(os.sched_getaffinity(0))
+    cpus = tuple(allowed[:2])
+    with relay_buffer(relay_cpu_affinity=cpus, workers=2, enable_graph=True) as buffer:
+        diagnostics = buffer.runtime.relay_diagnostics()
+        for worker in diagnostics["workers"]:
+            if worker["numa_node"] == 0:
+                assert worker["cpu"] in cpus, worker
+            else:
+                assert worker["cpu"] == -1, worker
+        assert [entry["bound"] for entry in diagnostics["replica_payload_placement"]] == [True, False]
+        inputs = make_inputs(WORLD, [TMAX] * WORLD, 1024, EXPERTS, TOPK, "random", seed=77)
+        result, (x, idx, weights) = run_dispatch(buffer, inputs, expand=True, capture=True)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False, rank_numa_nodes=TWO_SOCKETS)
+        cache = buffer.cache_layout(result[3])
+        del result
+        cached, _ = run_dispatch(buffer, inputs, expand=True, handle=cache, capture=True)
+        verify_dispatch(cached, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False, rank_numa_nodes=TWO_SOCKETS)
+        verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, TOPK)
+        del cached
+        graph = buffer.capture_dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
+        for _ in range(3):
+            for source in range(1, WORLD):
+                buffer.peers.set_source(source, *inputs[source])
+            buffer.peers.start(1, capture=True)
+            replayed = graph.replay()
+            torch.cuda.synchronize()
+            buffer.peers.wait(30_000)
+            verify_dispatch(replayed, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False, rank_numa_nodes=TWO_SOCKETS)
+            verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, TOPK)
+            del replayed
+
+
 def test_relay_delay_hook_requires_relay_mode():
     from test_gpu_dispatch import make_buffer
 

@@ -93,6 +93,38 @@ def test_static_scratch_matches_ordinary_dispatch(expand):
         assert_same(*dispatch_both_ways(buffer, small if expand else make_inputs(WORLD, [64] * WORLD, HIDDEN, EXPERTS, TOPK, "hotspot", seed=43), expand, 1))
 
 
+def test_static_scratch_dispatch_captured_into_a_graph():
+    """The entry point exists for callers under graph capture: its clearing step is
+    a fill kernel, not a memset node.  The dispatch is captured with a cached
+    layout and replayed several times, with eager dispatches of the ordinary entry
+    point (which leave other contents in the shared structures) in between; every
+    replay is compared with the oracle."""
+    inputs = make_inputs(WORLD, [128] * WORLD, HIDDEN, EXPERTS, TOPK, "random", seed=51)
+    other = make_inputs(WORLD, [90] * WORLD, HIDDEN, EXPERTS, TOPK, "multicast", seed=52)
+    with make_buffer(128, enable_graph=True) as buffer:
+        result, (x, idx, weights) = run_dispatch(buffer, inputs, expand=True)
+        verify_dispatch(result, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
+        cache = buffer.cache_layout(result[3])
+        del result
+        buffer.runtime.use_static_scratch = True
+        graph = buffer.capture_dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
+        buffer.runtime.use_static_scratch = False
+        for replay in range(4):
+            print(f"  replay {replay} of the captured static-scratch dispatch", flush=True)
+            for source in range(1, WORLD):
+                buffer.peers.set_source(source, *inputs[source])
+            buffer.peers.start(1, capture=True)
+            replayed = graph.replay()
+            torch.cuda.synchronize()
+            buffer.peers.wait(30_000)
+            verify_dispatch(replayed, inputs, 0, WORLD, EXPERTS, TOPK, True, 1, False)
+            verify_captured(buffer.peers, inputs, 0, WORLD, EXPERTS, TOPK)
+            del replayed
+            eager, _ = run_dispatch(buffer, other, expand=bool(replay % 2))
+            verify_dispatch(eager, other, 0, WORLD, EXPERTS, TOPK, bool(replay % 2), 1, False)
+            del eager
+
+
 def test_static_scratch_rejects_oversized_configuration():
     """4096 experts with 8192 tokens need more prologue scratch than the array holds."""
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
