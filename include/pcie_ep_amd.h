@@ -49,13 +49,13 @@ typedef struct pcie_ep_config {
     int32_t wire_fp8;           /* 0 BF16 wire, 1 E4M3FN + FP32 scale per token */
     int32_t timeout_ms;         /* device-side protocol timeout */
     int32_t fuse_receive_expand;/* 1: receive waves scatter to expert rows; 0: unique rows + expand kernel */
-    int32_t tx_waves;           /* payload TX wavefronts per payload workgroup, 0 = default (2) */
-    int32_t rx_waves;           /* payload RX wavefronts per payload workgroup, 0 = default (2; 4 on the FP8 wire) */
+    int32_t tx_waves;           /* tx_waves + rx_waves = payload wavefronts per payload workgroup, 0 = default (2 each). */
+    int32_t rx_waves;           /* The kernel decides row by row which direction a wavefront serves; the two values only add up. */
     int32_t peer_threads;       /* host threads standing in for the other ranks; 0 = none */
     int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
     int32_t device;             /* HIP device ordinal */
     int32_t worker_groups;      /* payload workgroups of the transport kernel, spread over the XCDs;
-                                   0 = default (48; 64 on the FP8 wire), -1 = none (control workgroups move the rows) */
+                                   0 = default (96), -1 = none (control workgroups move the rows) */
     int32_t receive_expand_mode;/* 0 pipelined, 1 vectorized, 2 scalar (pcie_ep/config.py:58-60): selects what the
                                    receive_expand_overlap diagnostic holds, the rows are moved the same way */
     int32_t numa_mode;          /* 0 direct; 1 relay: ranks on another NUMA domain are reached through host relay

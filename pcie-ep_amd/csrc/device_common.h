@@ -213,6 +213,17 @@ template <typename T>
 __device__ __forceinline__ T host_field_load(const T* address) {
     return __hip_atomic_load(address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
+// The same for an address the compiler cannot trace back to a kernel argument
+// (one rebuilt from lane shuffles, say): stating the global address space keeps
+// the access a global load instead of a flat one.
+__device__ __forceinline__ uint64_t host_load_global(const uint64_t* address) {
+    typedef const uint64_t __attribute__((address_space(1))) * GlobalWord;
+    return __hip_atomic_load((GlobalWord)address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ int32_t host_field_load_global(const int32_t* address) {
+    typedef const int32_t __attribute__((address_space(1))) * GlobalWord;
+    return __hip_atomic_load((GlobalWord)address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 template <typename T>
 __device__ __forceinline__ void host_field_store(T* address, T value) {
     __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);

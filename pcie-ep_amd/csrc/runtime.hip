@@ -134,19 +134,16 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
 }
 
 // Launch shape of the transport kernel: explicit values win, 0 selects the
-// measured defaults.  FP8 rows are half as long, so twice the RX wavefronts keep
-// the same bytes in flight, and a third more payload workgroups carry them
-// (T=8192: 5.16 ms against 5.28 ms with the BF16 shape).
+// defaults, which are the same for both wire formats.
 struct LaunchShape {
     int tx_waves, rx_waves, worker_groups;
 };
 LaunchShape resolve_launch_shape(const pcie_ep_config& c) {
     LaunchShape shape{};
     shape.tx_waves = c.tx_waves ? c.tx_waves : kDefaultTxWaves;
-    shape.rx_waves = c.rx_waves ? c.rx_waves : (c.wire_fp8 ? 2 * kDefaultRxWaves : kDefaultRxWaves);
+    shape.rx_waves = c.rx_waves ? c.rx_waves : kDefaultRxWaves;
     if (c.worker_groups < 0) shape.worker_groups = 0;
-    else if (c.worker_groups) shape.worker_groups = c.worker_groups;
-    else shape.worker_groups = c.wire_fp8 ? kDefaultWorkerGroups + kDefaultWorkerGroups / 3 : kDefaultWorkerGroups;
+    else shape.worker_groups = c.worker_groups ? c.worker_groups : kDefaultWorkerGroups;
     return shape;
 }
 

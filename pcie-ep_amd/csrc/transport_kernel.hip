@@ -31,10 +31,14 @@
 //    every control-path read, from the number of channels.
 //  * Workers publish their own descriptors and payload ACKs as soon as their own
 //    stores / loads have completed; control wavefronts only reserve and hand out.
-//  * A payload wavefront has a home direction (transmit or receive) but is not
-//    bound to it: once every ticket of its own direction has been claimed it
-//    takes tickets of the other one, so both directions end together whatever
-//    the routing's send/receive ratio is.
+//  * A payload wavefront has no fixed direction: before every row it takes the
+//    direction that needs it, in proportion to the rows left to send and to
+//    receive, so that the writes are spread thinly over the whole dispatch (row
+//    writes compete with the read REQUESTS for the upstream half of the link) and
+//    both directions end together whatever the routing's send/receive ratio is.
+//  * Vector memory operations complete in order: wherever several host words are
+//    wanted at once (count mailboxes, ACK arrays), their addresses are computed
+//    first and the loads issued in one run, with no other load in between.
 //  * Every read from host memory is a whole 16-byte vector per lane (payload, slot
 //    metadata, descriptor entries) or a packed word array (ACKs): small scattered
 //    reads cost the host link far more than their bytes.
@@ -135,10 +139,39 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     // written through to device memory (so no cache write-back is needed), and
     // ordering is by waiting for this wavefront's own operations.  A cache
     // write-back here would have to flush the rows the scatter is writing.
+    // Once every source's counts are ready, every mailbox word this wavefront needs
+    // is requested before the first one is used: one round trip over the host link
+    // instead of one per group.  Vector memory operations complete in order, so
+    // nothing else may be loaded in between - not even a segment's base address out of the kernel arguments:
+    // waiting for that load would wait for every host word requested before it.
+    // The addresses are therefore computed first (lane r holds the base of rank
+    // r's segment and hands it out by lane shuffle) - before the wait for the
+    // sources, where it costs nothing - and the loads follow in one run.
+    const char* const lane_segment = state.seg[lane < ranks ? lane : 0];
+    const auto segment_of = [&](int rank) {
+        const uint64_t bits = reinterpret_cast<uint64_t>(lane_segment);
+        return reinterpret_cast<char*>(uint64_t(uint32_t(__shfl(int(uint32_t(bits)), rank))) | uint64_t(uint32_t(__shfl(int(uint32_t(bits >> 32)), rank))) << 32);
+    };
+    constexpr int kExpectedPerLane = kMaxChannels * kMaxRanks / kWave;
+    const int32_t* expected_address[kExpectedPerLane];
+#pragma unroll
+    for (int i = 0; i < kExpectedPerLane; ++i) {
+        const int index = lane + i * kWave;
+        const bool valid = index < channels * ranks;
+        char* segment = segment_of(valid ? index % ranks : 0);
+        expected_address[i] = valid ? mailbox_at(z, segment, me) + 1 + local + index / ranks : nullptr;
+    }
+    const int32_t* first_address[kMaxRanks];
+#pragma unroll
+    for (int source = 0; source < kMaxRanks; ++source) {
+        char* segment = segment_of(source < ranks ? source : 0);
+        first_address[source] = (source < ranks && lane < local) ? mailbox_at(z, segment, me) + 1 + lane : nullptr;
+    }
+    const int32_t* unique_address = lane < ranks ? mailbox_at(z, const_cast<char*>(lane_segment), me) : nullptr;
     // All sources are polled in parallel, one lane each.
     bool ready = lane >= ranks;
     while (true) {
-        if (!ready) ready = host_load(signal_at(state.seg[lane], z.counts_ready_offset)) == epoch;
+        if (!ready) ready = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset)) == epoch;
         if (__all(ready)) break;
         if (health.poll(state, lane)) {
             if (lane == 0) record_error(state, kErrCountsReadyWait);
@@ -146,21 +179,16 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
         }
         backoff();
     }
-    // Every mailbox word this wavefront needs is requested now, before the first
-    // one is used: one round trip over the host link instead of one per group.
+    wait_memory_ops();
+    compiler_barrier();
     int unique = 0;
-    if (lane < ranks) unique = host_field_load(mailbox_at(z, state.seg[lane], me));
-    constexpr int kExpectedPerLane = kMaxChannels * kMaxRanks / kWave;
+    if (unique_address) unique = host_field_load_global(unique_address);
     int expected_values[kExpectedPerLane];
 #pragma unroll
-    for (int i = 0; i < kExpectedPerLane; ++i) {
-        const int index = lane + i * kWave;
-        expected_values[i] = index < channels * ranks ? host_field_load(mailbox_at(z, state.seg[index % ranks], me) + 1 + local + index / ranks) : 0;
-    }
+    for (int i = 0; i < kExpectedPerLane; ++i) expected_values[i] = expected_address[i] ? host_field_load_global(expected_address[i]) : 0;
     int first_counts[kMaxRanks];
 #pragma unroll
-    for (int source = 0; source < kMaxRanks; ++source)
-        first_counts[source] = (source < ranks && lane < local) ? host_field_load(mailbox_at(z, state.seg[source], me) + 1 + lane) : 0;
+    for (int source = 0; source < kMaxRanks; ++source) first_counts[source] = first_address[source] ? host_field_load_global(first_address[source]) : 0;
     // The reads are on the link (requests leave in issue order): the receive side
     // may now flood it with row reads without delaying these few words.
     compiler_barrier();
@@ -372,23 +400,46 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
         if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
         if (workers_finished && !drained) {
-            // Each pass checks up to 64 / endpoints ordinals of every endpoint; lanes of
-            // one endpoint read consecutive ACK words (one 64-byte read per eight slots).
+            // Each pass checks up to kDrainBatch * (64 / endpoints) ordinals of every
+            // endpoint; lanes of one endpoint read consecutive ACK words (one 64-byte read
+            // per eight slots) and all reads of a pass are on the link before the first
+            // is used, so a ring window costs a few round trips, not one per handful of slots.
             // While the channel's receive side is still busy the drain is not what the
             // kernel waits for: it then polls sparingly, so that the small reads do not
             // compete with the row reads for the link.
             const bool receive_busy = broadcast_first(int(device_load(&q.rx_finished[channel].value))) == 0;
             if (!receive_busy || broadcast_first(now_ticks() >= next_drain_poll ? 1 : 0)) {
-                const int per_pass = kWave / endpoints;
-                const int my_ordinal = drain_ordinal + lane % per_pass;
-                const int endpoint = lane / per_pass;
-                int missing_ordinal = 0x7FFFFFFF;
-                if (endpoint < endpoints && my_ordinal < produced) {
-                    const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
-                    const uint32_t remote = endpoint_mask_of(z.dims, me, state.plan_mask[token]);
-                    if (((remote >> endpoint) & 1u) && host_load(ack_at(z, own, channel, my_ordinal % slots, endpoint)) != sequence(epoch, token))
-                        missing_ordinal = my_ordinal;
+                constexpr int kDrainBatch = 8;
+                const int group = kWave / endpoints;
+                const int per_pass = group * kDrainBatch;
+                const int endpoint = lane / group;
+                // Vector memory operations complete in order: what the ACK addresses depend
+                // on (tokens, route masks) is loaded first, the host reads follow in one run.
+                uint64_t seen[kDrainBatch], wanted[kDrainBatch];
+                const uint64_t* address[kDrainBatch];
+#pragma unroll
+                for (int batch = 0; batch < kDrainBatch; ++batch) {
+                    const int my_ordinal = drain_ordinal + batch * group + lane % group;
+                    seen[batch] = wanted[batch] = 0;
+                    address[batch] = nullptr;
+                    if (endpoint < endpoints && my_ordinal < produced) {
+                        const int token = device_load(state.chan_remote_tokens + size_t(channel) * stride + my_ordinal);
+                        const uint32_t remote = endpoint_mask_of(z.dims, me, state.plan_mask[token]);
+                        if ((remote >> endpoint) & 1u) {
+                            wanted[batch] = sequence(epoch, token);
+                            address[batch] = ack_at(z, own, channel, my_ordinal % slots, endpoint);
+                        }
+                    }
                 }
+                wait_memory_ops();
+                compiler_barrier();
+#pragma unroll
+                for (int batch = 0; batch < kDrainBatch; ++batch)
+                    if (address[batch]) seen[batch] = host_load_global(address[batch]);
+                int missing_ordinal = 0x7FFFFFFF;
+#pragma unroll
+                for (int batch = kDrainBatch - 1; batch >= 0; --batch)
+                    if (seen[batch] != wanted[batch]) missing_ordinal = drain_ordinal + batch * group + lane % group;
                 for (int offset = 32; offset > 0; offset >>= 1) {
                     const int other = __shfl_xor(missing_ordinal, offset);
                     missing_ordinal = other < missing_ordinal ? other : missing_ordinal;
@@ -1003,20 +1054,45 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 // ---------------------------------------------------------------------------------------
 // Payload wavefront: moves rows of either direction
 // ---------------------------------------------------------------------------------------
-// Every payload wavefront has a home direction (the first tx_waves wavefronts of
-// a workgroup transmit, the others receive) and serves it until every ticket of
-// that direction has been claimed.  Then, instead of leaving, it takes tickets
-// of the other direction: the two directions end together whatever the
-// routing's send/receive ratio is, and the split only sets how the link is shared
-// while both have work.  A ticket of the other direction is only claimed when
-// its producer has already reserved it (head < tail), so a wavefront never
-// commits itself to a row that does not exist yet.
+// A payload wavefront serves whichever direction needs it.  The two directions
+// share the host link: row reads return on the downstream half, but their
+// requests travel upstream beside the row writes, so a transmit side that runs
+// flat out (about 24 GB/s next to saturated reads) takes request slots from the
+// receive side (55 instead of 57 GB/s) and is then idle for the rest of the
+// dispatch.  The wavefronts therefore split in proportion to the work that is
+// LEFT in each direction: with rem_tx and rem_rx rows still unclaimed,
+//     transmitting wavefronts : receiving wavefronts = kTxWeight * rem_tx : kRxWeight * (rem_rx - lead)
+// (one wavefront's share of the link's write rate is about 4/9 of its share of
+// the read rate), re-evaluated before every row, so the writes are spread
+// thinly over the whole dispatch whatever the routing's send/receive ratio is.
+// `lead` makes the transmit side end a little earlier than the receive side (by
+// the time the link needs for kTxLeadBytes): a transmitted row is only finished
+// when its receivers have acknowledged it, and that round trip then hides
+// behind the last received rows instead of following them.  The rule corrects
+// itself: a direction that falls behind has more left and gets more wavefronts;
+// at most half of the wavefronts transmit and, while anything is left to send, at
+// least kMinTxWaves.  Until both totals are known (the receive total comes with
+// the receive prefixes) those kMinTxWaves transmit and everybody else waits for
+// the first descriptors.  A wavefront whose direction has nothing to
+// claim takes a ticket of the other direction instead - at once when its own
+// direction is finished, after kIdleCrossoverUs otherwise (at the start of a
+// dispatch the first descriptors are a few microseconds away and a receive
+// wavefront must not bind itself to a transmit row for them) - but only a
+// ticket its producer has already reserved (head < tail), so it never commits
+// itself to a row that does not exist yet.
+constexpr int64_t kTxWeight = 9, kRxWeight = 4;
+constexpr int64_t kTxLeadBytes = 24 << 20;
+constexpr int kMinTxWaves = 16;
+constexpr uint64_t kIdleCrossoverUs = 30;
+
 template <bool kFp8, bool kVector>
-__device__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, bool home_tx) {
+__device__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int order, int waves) {
     const uint64_t epoch = *state.epoch;
     Deadline deadline(now_ticks());
     WorkerCounters counters;
     bool prefixes_known = false;
+    const int lead = int(kTxLeadBytes / int64_t(state.z.meta_offset + state.z.meta_bytes));
+    uint64_t idle_since = 0;  // 0: the last look found work
     while (true) {
         // 0: nothing to do now, 1: transmit, 2: receive, -1: both directions are finished or the kernel aborts.
         int choice = 0;
@@ -1028,9 +1104,25 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
                 const bool rx_backlog = rx_head < int(device_load(&q.rx_tail.value));
                 const int tx_total = device_load(&q.tx_head.total), rx_total = device_load(&q.rx_head.total);
                 const bool tx_done = tx_total >= 0 && tx_head >= tx_total, rx_done = rx_total >= 0 && rx_head >= rx_total;
-                if (home_tx ? tx_backlog : rx_backlog) choice = home_tx ? 1 : 2;
-                else if ((home_tx ? tx_done : rx_done) && (home_tx ? rx_backlog : tx_backlog)) choice = home_tx ? 2 : 1;
-                if (choice == 0) {
+                // Totals unknown: a handful of wavefronts start to transmit, the others
+                // wait for the first descriptors.
+                bool prefer_tx = order < kMinTxWaves;
+                if (tx_total >= 0 && rx_total >= 0) {
+                    const int rx_rows = rx_total - rx_head - lead;
+                    const int64_t tx_left = tx_done ? 0 : kTxWeight * (tx_total - tx_head), rx_left = rx_rows > 0 ? kRxWeight * rx_rows : 0;
+                    prefer_tx = rx_done || (tx_left > 0 && 2 * order < waves &&
+                                            (order < kMinTxWaves || int64_t(order) * (tx_left + rx_left) < int64_t(waves) * tx_left));
+                }
+                const bool own_backlog = prefer_tx ? tx_backlog : rx_backlog, other_backlog = prefer_tx ? rx_backlog : tx_backlog;
+                const bool own_done = prefer_tx ? tx_done : rx_done;
+                if (own_backlog) choice = prefer_tx ? 1 : 2;
+                else if (other_backlog) {
+                    const uint64_t now = now_ticks();
+                    if (!idle_since) idle_since = now;
+                    if (own_done || now - idle_since > kIdleCrossoverUs * state.clock_khz / 1000) choice = prefer_tx ? 2 : 1;
+                }
+                if (choice) idle_since = 0;
+                else {
                     if (tx_done && rx_done) choice = -1;
                     else if (deadline.expired(state)) {
                         record_error(state, kErrRingProgressWait);
@@ -1105,7 +1197,11 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
         wave -= 2;
     }
     if (wave >= payload_waves) return;
-    payload_worker<kFp8, kVector>(state, q, scratch, lane, wave < state.tx_waves);
+    // Position of this wavefront among all payload wavefronts, wavefront-major: a
+    // direction's share is spread over the workgroups before it doubles up in one.
+    const int groups = payload_groups ? payload_groups : channels;
+    const int group = payload_groups ? block - channels : block;
+    payload_worker<kFp8, kVector>(state, q, scratch, lane, wave * groups + group, groups * payload_waves);
     finish_role(state, q, lane, roles);
     // Every role loop has an explicit completion, abort or timeout exit and no
     // workgroup barrier follows the entry verdict.

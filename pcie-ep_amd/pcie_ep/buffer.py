@@ -150,9 +150,10 @@ class HostStagedEPBuffer:
         plays; ``peer_threads`` the host threads standing in for the others
         (default: one per peer, at most 7); ``staging_numa_node`` binds the pinned
         rings to a NUMA node; ``worker_groups`` / ``tx_waves`` / ``rx_waves``
-        shape the transport kernel (0 = defaults: 48 payload workgroups of 2 TX +
-        2 RX wavefronts; 64 of 2 TX + 4 RX on the FP8 wire; ``worker_groups=-1`` makes the
-        per-channel control workgroups move the rows themselves).
+        shape the transport kernel (0 = defaults: 96 payload workgroups of 2 + 2
+        wavefronts on either wire; which direction a wavefront serves is decided
+        inside the kernel, only the sum of the two numbers matters; ``worker_groups=-1`` makes the per-channel control
+        workgroups move the rows themselves).
         ``rank_numa_nodes`` (relay mode) gives the NUMA node of every logical rank,
         which the reference gathers from its processes; ranks of another node than
         a source's are reached through that source's relay workers and replica
