@@ -55,7 +55,8 @@ typedef struct pcie_ep_config {
     int32_t staging_numa_node;  /* NUMA node for the pinned segments, -1 = first touch */
     int32_t device;             /* HIP device ordinal */
     int32_t worker_groups;      /* payload workgroups of the transport kernel, spread over the XCDs;
-                                   0 = default (96), -1 = none (control workgroups move the rows) */
+                                   0 = default (as many as keep 2.7 MB of rows in flight: 48 for 14 KB rows, at most 96),
+                                   -1 = none (control workgroups move the rows) */
     int32_t receive_expand_mode;/* 0 pipelined, 1 vectorized, 2 scalar (pcie_ep/config.py:58-60): selects what the
                                    receive_expand_overlap diagnostic holds, the rows are moved the same way */
     int32_t numa_mode;          /* 0 direct; 1 relay: ranks on another NUMA domain are reached through host relay
@@ -285,7 +286,7 @@ int pcie_ep_measure_kernel_host_copy(int32_t device, int64_t bytes, int32_t repe
  * No counterpart in the reference. */
 int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, double* gbps);
 
-/* Read+write rate (GB/s, best of `repeats`) of the expand kernel's traffic shape
+/* Read+write rate (GB/s; best of three batches of `repeats` back-to-back launches) of the expand kernel's traffic shape
  * without its metadata: every wavefront reads one row of `row_bytes` and writes
  * it once, `extra_per_1024` of every 1024 rows twice.  pattern 0 writes in linear
  * order, 1 into `streams` interleaved sequential streams (what expert-major

@@ -10,12 +10,16 @@ namespace pcie_ep {
 // Payload workgroups of the transport kernel (after the C control workgroups)
 // and the payload wavefronts each of them carries (tx_waves + rx_waves: which
 // direction a wavefront serves is decided row by row inside the kernel, so only
-// the sum of the two numbers matters).  Every wavefront has
-// one row in flight, so their number sets the bytes outstanding on the host
-// link: 384 wavefronts keep a Gen5 x16 link saturated with 7 KB (FP8) as well
-// as 14 KB (BF16) rows; measured at T=8192, 48 to 96 workgroups are within
-// 0.2 % of each other on the BF16 wire and 96 are 1.5 % faster than 64 on FP8.
-constexpr int kDefaultWorkerGroups = 96;
+// the sum of the two numbers matters).  Every wavefront has one row in flight, so
+// their number sets the bytes outstanding on the host link.  The default keeps
+// kBytesInFlight outstanding whatever the row size is: 48 workgroups of four
+// wavefronts for 14 KB rows (BF16, hidden 7168), 96 for 7 KB rows (the FP8 wire:
+// measured 1.5 % faster than 64) and for anything shorter.  More wavefronts than
+// that buy nothing on the link (48 to 96 workgroups are within 0.2 % of each
+// other for 14 KB rows) and take compute units from kernels running beside the
+// dispatch.
+constexpr int64_t kBytesInFlight = 2736 << 10;
+constexpr int kMinDefaultWorkerGroups = 16, kMaxDefaultWorkerGroups = 96;
 constexpr int kDefaultTxWaves = 2;
 constexpr int kDefaultRxWaves = 2;
 constexpr int kMaxTxWaves = 4;

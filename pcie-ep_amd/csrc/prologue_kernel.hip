@@ -90,7 +90,10 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     __shared__ int stalled;
     if (threadIdx.x == 0) stalled = 0;
 
-    bool aborted = false, consumed = true;
+    // Direct mode has at most kMaxRanks * (1 + kMaxChannels) = 528 abort words, a workgroup at least 256 threads.
+    constexpr int kAbortLoadsPerThread = 3;
+    uint64_t abort_words[kAbortLoadsPerThread] = {0, 0, 0};
+    uint64_t consumed_word = tag - 1;
     if (leader) {
         // ---- begin epoch: clear per-dispatch diagnostics -----------------------------
         for (int i = threadIdx.x; i < kErrorFields; i += blockDim.x) state.errors[i] = 0;
@@ -118,13 +121,19 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
             q.rx_retired[i].total = q.tx_retired[i].total = q.rx_finished[i].total = -1;
         }
         // Abort signals are terminal, and the previous count mailbox must have
-        // been consumed.  Issue the host loads now; the verdicts are taken after
-        // the layout so their PCIe latency hides behind it.
+        // been consumed.  The host loads are only issued here: their values are
+        // first looked at after the layout, so the round trip over the host link
+        // hides behind it (a use right here would make every thread wait for it).
         const int per_rank = abort_flags_per_rank(z);
-        for (int index = threadIdx.x; index < ranks * per_rank; index += blockDim.x)
-            aborted |= host_load(abort_flag_at(z, state.seg[index / per_rank], index % per_rank)) != 0;
-        if (wave == 0 && tag > 1 && lane < ranks && lane != state.local_rank)
-            consumed = host_load(signal_at(own, z.counts_consumed_offset, lane)) == tag - 1;
+#pragma unroll
+        for (int i = 0; i < kAbortLoadsPerThread; ++i) {
+            const int index = threadIdx.x + i * int(blockDim.x);
+            if (index < ranks * per_rank) abort_words[i] = host_load(abort_flag_at(z, state.seg[index / per_rank], index % per_rank));
+        }
+        // (Relay mode with many domains has more flags than that: the rest is read the plain way.)
+        for (int index = threadIdx.x + kAbortLoadsPerThread * int(blockDim.x); index < ranks * per_rank; index += blockDim.x)
+            abort_words[0] |= host_load(abort_flag_at(z, state.seg[index / per_rank], index % per_rank));
+        if (wave == 0 && tag > 1 && lane < ranks && lane != state.local_rank) consumed_word = host_load(signal_at(own, z.counts_consumed_offset, lane));
     }
 
     // ---- stable layout ---------------------------------------------------------------
@@ -282,10 +291,16 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
                 if (key != 0x7FFFFFFF) record_error(state, kErrInvalidRouting, key / 64, key % 64);
             }
         }
-        __threadfence();
     }
 
     // ---- epoch verdict -----------------------------------------------------------------
+    // Everything the leader's threads hand to each other below (plan totals, the
+    // error record) stays inside this workgroup: the barriers order it, no cache
+    // write-back is needed before the kernel ends.
+    bool aborted = false;
+#pragma unroll
+    for (int i = 0; i < kAbortLoadsPerThread; ++i) aborted |= abort_words[i] != 0;
+    bool consumed = consumed_word == tag - 1;
     const bool any_abort = __syncthreads_or(aborted);
     if (threadIdx.x == 0) {
         *state.epoch = tag;
@@ -294,7 +309,6 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         else if (any_abort) record_error(state, kErrAlreadyAborted);
         // Any error here (including invalid routing found above) is terminal for this buffer.
         if (load_error_code(state)) host_store_release(signal_at(own, z.channel_abort_offset), tag);
-        __threadfence();
     }
     __syncthreads();
     const uint64_t epoch = tag;

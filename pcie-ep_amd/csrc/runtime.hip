@@ -134,7 +134,9 @@ int check_config(const pcie_ep_config* c, Dimensions& dims) {
 }
 
 // Launch shape of the transport kernel: explicit values win, 0 selects the
-// defaults, which are the same for both wire formats.
+// defaults.  The default number of payload workgroups follows from the row size
+// alone (a fixed number of bytes in flight on the host link), in steps of eight
+// so that every XCD gets the same number.
 struct LaunchShape {
     int tx_waves, rx_waves, worker_groups;
 };
@@ -143,7 +145,15 @@ LaunchShape resolve_launch_shape(const pcie_ep_config& c) {
     shape.tx_waves = c.tx_waves ? c.tx_waves : kDefaultTxWaves;
     shape.rx_waves = c.rx_waves ? c.rx_waves : kDefaultRxWaves;
     if (c.worker_groups < 0) shape.worker_groups = 0;
-    else shape.worker_groups = c.worker_groups ? c.worker_groups : kDefaultWorkerGroups;
+    else if (c.worker_groups) shape.worker_groups = c.worker_groups;
+    else {
+        const int64_t row_bytes = int64_t(c.hidden) * (c.wire_fp8 ? 1 : 2) + 256;  // payload + slot metadata, roughly
+        const int64_t waves = (kBytesInFlight + row_bytes - 1) / row_bytes;
+        const int64_t per_group = shape.tx_waves + shape.rx_waves;
+        int64_t groups = ((waves + per_group - 1) / per_group + 7) / 8 * 8;
+        groups = groups < kMinDefaultWorkerGroups ? kMinDefaultWorkerGroups : groups;
+        shape.worker_groups = int(groups > kMaxDefaultWorkerGroups ? kMaxDefaultWorkerGroups : groups);
+    }
     return shape;
 }
 
@@ -223,7 +233,7 @@ struct pcie_ep_runtime {
     char* segments[kMaxRanks] = {};
     uint64_t* epoch = nullptr;
     int32_t* chan_remote_tokens = nullptr;
-    int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves, worker_groups = kDefaultWorkerGroups;
+    int tx_waves = kDefaultTxWaves, rx_waves = kDefaultRxWaves, worker_groups = kMinDefaultWorkerGroups;
     TransportQueues* queues = nullptr;
     char* layout_scratch = nullptr;
     uint64_t metadata_delay = 0, tx_delay = 0, rx_delay = 0, scatter_delay = 0, prefix_delay = 0, control_abort_after = 0;
@@ -830,16 +840,19 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
     if (status == hipSuccess) status = hipStreamCreate(&stream);
     if (status == hipSuccess) status = hipEventCreate(&begin);
     if (status == hipSuccess) status = hipEventCreate(&end);
+    // One untimed launch, then three batches of `repeats` back-to-back launches
+    // between one pair of events each (no event or launch-gap overhead per launch).
     double best = 0.0;
-    for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+    if (status == hipSuccess) status = launch_copy(source, destination, bytes, stream);
+    for (int batch = 0; batch < 3 && status == hipSuccess; ++batch) {
         status = hipEventRecord(begin, stream);
-        if (status == hipSuccess) status = launch_copy(source, destination, bytes, stream);
+        for (int i = 0; i < repeats && status == hipSuccess; ++i) status = launch_copy(source, destination, bytes, stream);
         if (status == hipSuccess) status = hipEventRecord(end, stream);
         if (status == hipSuccess) status = hipEventSynchronize(end);
         float ms = 0.0f;
         if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
-        if (status == hipSuccess && i > 0 && ms > 0.0f) {
-            const double rate = 2.0 * double(bytes) / (ms * 1e6);  // bytes read + bytes written
+        if (status == hipSuccess && ms > 0.0f) {
+            const double rate = 2.0 * double(bytes) * repeats / (ms * 1e6);  // bytes read + bytes written
             if (rate > best) best = rate;
         }
     }
@@ -872,18 +885,23 @@ int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes,
     // Rows written twice, counted exactly as the kernel selects them.
     int64_t twice = 0;
     for (int row = 0; row < rows; ++row) twice += (row & 1023) * extra_per_1024 / 1024 != ((row & 1023) + 1) * extra_per_1024 / 1024;
+    // One untimed launch, then three batches of `repeats` back-to-back launches
+    // between one pair of events each: the per-launch mean of a batch carries no
+    // event or launch-gap overhead (a tenth of a 100 us kernel otherwise).
     double best = 0.0;
-    for (int i = 0; i <= repeats && status == hipSuccess; ++i) {  // first iteration warms up
+    if (status == hipSuccess) status = launch_row_scatter(source, destination, rows, row_bytes, extra_per_1024, pattern, streams, stream);
+    for (int batch = 0; batch < 3 && status == hipSuccess; ++batch) {
         status = hipEventRecord(begin, stream);
-        if (status == hipSuccess) status = launch_row_scatter(source, destination, rows, row_bytes, extra_per_1024, pattern, streams, stream);
+        for (int i = 0; i < repeats && status == hipSuccess; ++i)
+            status = launch_row_scatter(source, destination, rows, row_bytes, extra_per_1024, pattern, streams, stream);
         if (status == hipSuccess) status = hipEventRecord(end, stream);
         if (status == hipSuccess) status = hipEventSynchronize(end);
         float ms = 0.0f;
         if (status == hipSuccess) status = hipEventElapsedTime(&ms, begin, end);
-        if (status == hipSuccess && i > 0 && ms > 0.0f) {
+        if (status == hipSuccess && ms > 0.0f) {
             // bytes read + bytes written; the read-only and write-only patterns move every row once
             const double moved = pattern >= 3 ? double(rows) : double(2 * int64_t(rows) + twice);
-            const double rate = moved * double(row_bytes) / (ms * 1e6);
+            const double rate = moved * double(row_bytes) * repeats / (ms * 1e6);
             if (rate > best) best = rate;
         }
     }

@@ -150,8 +150,9 @@ class HostStagedEPBuffer:
         plays; ``peer_threads`` the host threads standing in for the others
         (default: one per peer, at most 7); ``staging_numa_node`` binds the pinned
         rings to a NUMA node; ``worker_groups`` / ``tx_waves`` / ``rx_waves``
-        shape the transport kernel (0 = defaults: 96 payload workgroups of 2 + 2
-        wavefronts on either wire; which direction a wavefront serves is decided
+        shape the transport kernel (0 = defaults: payload workgroups of 2 + 2
+        wavefronts, as many as keep 2.7 MB of rows in flight - 48 for BF16 rows of
+        hidden 7168, 96 on the FP8 wire; which direction a wavefront serves is decided
         inside the kernel, only the sum of the two numbers matters; ``worker_groups=-1`` makes the per-channel control
         workgroups move the rows themselves).
         ``rank_numa_nodes`` (relay mode) gives the NUMA node of every logical rank,
