@@ -75,6 +75,23 @@ def test_full_hidden_32_channels():
         check_case(buffer, "h7168-gpu-empty", [0] + [129] * 7, seed=10)
 
 
+def test_lopsided_send_receive_ratios():
+    """A payload wavefront chooses its direction by the rows left to send and to
+    receive: the extremes (nothing to receive, nothing to send, hundreds of rows
+    one way against a handful the other way) must end like any other dispatch,
+    also with rings that wrap many times and with the default launch shape."""
+    with make_buffer(tmax=1500, channels=8, hidden=1024, payload_slots=16, descriptor_slots=16) as buffer:
+        check_case(buffer, "send-only", [1500] + [0] * 7, capture=True)
+        check_case(buffer, "receive-only", [0] + [1500] * 7)
+        check_case(buffer, "send-heavy", [1500] + [3] * 7, capture=True, seed=21)
+        check_case(buffer, "receive-heavy", [2] + [1500] * 7, capture=True, seed=22)
+        check_case(buffer, "send-heavy-multicast", [1500] + [1] * 7, "multicast", expand=False, seed=23)
+        check_case(buffer, "one-source", [40, 0, 0, 1500, 0, 0, 0, 0], seed=24)
+    with make_buffer(tmax=1500, channels=8, hidden=1024, stage=7, wire_dtype="fp8_e4m3") as buffer:
+        check_case(buffer, "fp8-send-heavy", [1500] + [5] * 7, capture=True, seed=25, fp8=True)
+        check_case(buffer, "fp8-receive-heavy", [4] + [1500] * 7, seed=26, fp8=True)
+
+
 @pytest.mark.parametrize("rank", [3, 7])
 def test_other_local_rank(rank):
     with make_buffer(rank=rank, channels=3, hidden=512, payload_slots=4, descriptor_slots=4) as buffer:
