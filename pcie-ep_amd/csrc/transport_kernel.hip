@@ -148,6 +148,10 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     // r's segment and hands it out by lane shuffle) - before the wait for the
     // sources, where it costs nothing - and the loads follow in one run.
     const char* const lane_segment = state.seg[lane < ranks ? lane : 0];
+    // The first look at every source's counts_ready is requested now; its value is
+    // used after the address arithmetic below, which so runs inside its round trip.
+    uint64_t first_look = 0;
+    if (lane < ranks) first_look = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
     const auto segment_of = [&](int rank) {
         const uint64_t bits = reinterpret_cast<uint64_t>(lane_segment);
         return reinterpret_cast<char*>(uint64_t(uint32_t(__shfl(int(uint32_t(bits)), rank))) | uint64_t(uint32_t(__shfl(int(uint32_t(bits >> 32)), rank))) << 32);
@@ -169,8 +173,9 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     }
     const int32_t* unique_address = lane < ranks ? mailbox_at(z, const_cast<char*>(lane_segment), me) : nullptr;
     // All sources are polled in parallel, one lane each.
-    bool ready = lane >= ranks;
+    bool ready = lane >= ranks || first_look == epoch;
     while (true) {
+        if (__all(ready)) break;
         if (!ready) ready = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset)) == epoch;
         if (__all(ready)) break;
         if (health.poll(state, lane)) {
@@ -501,21 +506,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     const bool replica = member && reads_replica(z.dims, source, me);
     const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
     int expected = member ? 0x7FFFFFFF : 0, total = 0x7FFFFFFF;
-    bool counts_known = false, prefix_failed = false;
-    // ... but not before the producer of the prefixes has requested the count
-    // mailboxes: a few hundred bytes that everything waits for must not queue
-    // behind megabytes of row reads.
-    while (true) {
-        int gate = 0;
-        if (lane == 0) gate = (device_load(state.receive_prefix_state) & kPrefixRequested) ? 1 : (aborted(q) ? -1 : 0);
-        gate = broadcast_first(gate);
-        if (gate > 0) break;
-        if (gate < 0 || receive_prefix_verdict(state, epoch, lane) < 0) {
-            prefix_failed = true;
-            break;
-        }
-        backoff();
-    }
+    bool counts_known = false, prefix_failed = false, gate_open = false;
     const uint64_t below = lanes_below(lane);
     const uint64_t group_mask = (1ull << lookahead) - 1ull;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
@@ -561,6 +552,21 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             backoff();
             continue;
         }
+        // The descriptors are polled from the start (a few dozen bytes per source),
+        // but no row is handed out before the producer of the prefixes has requested
+        // the count mailboxes: a few hundred bytes that everything waits for must not
+        // queue behind megabytes of row reads.
+        while (!gate_open) {
+            int gate = 0;
+            if (lane == 0) gate = (device_load(state.receive_prefix_state) & kPrefixRequested) ? 1 : (aborted(q) ? -1 : 0);
+            gate = broadcast_first(gate);
+            if (gate > 0) gate_open = true;
+            else if (gate < 0 || receive_prefix_verdict(state, epoch, lane) < 0) {
+                prefix_failed = true;
+                break;
+            } else backoff();
+        }
+        if (prefix_failed) break;
         const int ticket_index = reserve_tickets(q.rx_tail, __popcll(accepted), lane) + __popcll(accepted & below);
         const int slot = int(published[2]), token = int(published[3]);
         const uint64_t payload_sequence = sequence(epoch, token);
