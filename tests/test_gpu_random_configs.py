@@ -66,3 +66,39 @@ def test_random_configurations(first):
                     verify_captured(buffer.peers, inputs, c["rank"], c["world"], c["experts"], c["topk"], fp8_wire=c["fp8"],
                                     with_weights=c["weights"])
                 del result
+
+
+@pytest.mark.parametrize("first", range(1000, 1040, 20))
+def test_random_configurations_through_the_relay(first):
+    """The same walk in NUMA relay mode (stage 8): a random map of the ranks onto
+    two to four NUMA domains and random replica ring sizes, so rows cross domains
+    in both directions through relay workers and replica rings of every shape."""
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    for case in range(first, first + 20):
+        c = draw(case)
+        if c["world"] == 1:
+            continue
+        rng = random.Random(case * 7 + 1)
+        domains = rng.randint(2, min(4, c["world"]))
+        nodes = tuple(rng.randrange(domains) for _ in range(c["world"]))
+        if len(set(nodes)) < 2:
+            nodes = tuple(index % 2 for index in range(c["world"]))
+        replica_slots = rng.choice([1, 2, 4, 16])
+        print(f"case {case}: {c} nodes={nodes} replica_slots={replica_slots}", flush=True)
+        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000, stage=8,
+                                  numa_mode="relay", replica_slots=replica_slots, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16",
+                                  fuse_receive_expand=c["fuse"], receive_expand_mode="pipelined" if c["fuse"] else "scalar")
+        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
+                                config=config, num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0], rx_waves=c["waves"][1],
+                                worker_groups=c["waves"][2], rank_numa_nodes=nodes) as buffer:
+            for repeat in range(2):
+                inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + repeat,
+                                     gaussian=c["fp8"], heavy_tail=c["fp8"])
+                result, _ = run_dispatch(buffer, inputs, expand=c["expand"], alignment=c["alignment"], zero_padding=c["expand"],
+                                         with_weights=c["weights"], capture=True)
+                verify_dispatch(result, inputs, c["rank"], c["world"], c["experts"], c["topk"], c["expand"], c["alignment"], c["expand"],
+                                with_weights=c["weights"], fp8_wire=c["fp8"], rank_numa_nodes=nodes)
+                verify_captured(buffer.peers, inputs, c["rank"], c["world"], c["experts"], c["topk"], fp8_wire=c["fp8"],
+                                with_weights=c["weights"])
+                del result
