@@ -297,6 +297,36 @@ int pcie_ep_measure_device_copy(int32_t device, int64_t bytes, int32_t repeats, 
 int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes, int32_t extra_per_1024, int32_t pattern, int32_t streams,
                                 int32_t repeats, double* gbps);
 
+/* Publication / acknowledgement litmus on the kind of memory the segments are
+ * made of (pinned, fine-grained, mapped), with the access primitives of the
+ * transport kernel: the experiment of the reference's stand-alone two-GPU
+ * program (tests/mapped_litmus.cu, tests/MAPPED_LITMUS.md - one payload slot,
+ * READY and ACK words 128 bytes apart, sequences from 1, a delayed last thread)
+ * between this GPU and the calling CPU thread.  mode 0: one wavefront produces,
+ * the CPU consumes; 1: a workgroup of four wavefronts produces; 2: the CPU
+ * produces, one wavefront consumes; 3: a workgroup consumes.  Every round the
+ * consumer compares every word of the payload with what the round must hold.
+ * Mode 0 or 1 with PCIE_EP_LITMUS_PUBLISH_EARLY added is the negative control:
+ * the producer publishes READY without waiting for its payload stores; with
+ * other traffic on the host link the consumer then finds stale words (code 4),
+ * which shows that the experiment can fail and that the wait is needed.
+ * Codes: 0 passed, 1 READY timeout, 2 ACK timeout, 3 the other side gave up,
+ * 4 payload mismatch (index = first bad 16-byte vector).  Every wait on either
+ * side is bounded by timeout_ms, so the kernel always ends. */
+#define PCIE_EP_LITMUS_PUBLISH_EARLY 16
+typedef struct pcie_ep_litmus_result {
+    int64_t completed;      /* rounds both sides completed without error (0 on any failure) */
+    int32_t gpu_code;       /* what the GPU side found */
+    int32_t host_code;      /* what the CPU side found */
+    int64_t gpu_iteration;  /* round of the GPU side's failure */
+    int64_t gpu_index;      /* vector of a mismatch the GPU side found, else -1 */
+    int64_t host_iteration;
+    int64_t host_index;
+    double seconds;         /* wall clock of all rounds */
+} pcie_ep_litmus_result;
+int pcie_ep_litmus(int32_t device, int32_t mode, int64_t iterations, int32_t payload_bytes, int32_t writer_delay_ns, int32_t reader_delay_ns,
+                   int32_t timeout_ms, pcie_ep_litmus_result* result);
+
 /* ---- Host peer emulator ---------------------------------------------------
  * On one GPU the other logical ranks are host threads that follow the ring
  * protocol on the same pinned segments, the way the reference's CPU relay

@@ -23,7 +23,7 @@ LIBRARY = OUT_DIR / "libpcie_ep_amd.so"
 CLIENT = OUT_DIR / "abi_client"
 OBJ_DIR = HERE / "build"
 
-HIP_SOURCES = ["prologue_kernel.hip", "transport_kernel.hip", "expand_kernels.hip", "runtime.hip"]
+HIP_SOURCES = ["prologue_kernel.hip", "transport_kernel.hip", "expand_kernels.hip", "litmus.hip", "runtime.hip"]
 CXX_SOURCES = ["peers.cpp", "relay.cpp"]
 
 COMMON = ["-O3", "-std=c++20", "-fPIC", "-Wall", "-Wno-unused-function", "-pthread"]

@@ -3,6 +3,10 @@
 
 #include <hip/hip_runtime.h>
 
+#include <string>
+
+#include "../../include/pcie_ep_amd.h"
+
 #include "device_common.h"
 
 namespace pcie_ep {
@@ -63,6 +67,9 @@ hipError_t launch_row_scatter(const void* source, void* destination, int rows, i
 hipError_t launch_zero(void* destination, size_t bytes, hipStream_t stream);
 // Kernel-driven copy between pinned host memory and HBM with `wavefronts` wavefronts in flight.
 hipError_t launch_host_copy(void* host, void* device, int64_t bytes, bool to_device, int wavefronts, hipStream_t stream);
+// Publication / acknowledgement litmus on pinned host memory (litmus.hip); 0 or a PCIE_EP_E_* code.
+int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int writer_delay_ns, int reader_delay_ns, int timeout_ms,
+               pcie_ep_litmus_result* out, std::string& error);
 // Stand-alone FP8 wire kernels.
 hipError_t launch_quantize(const uint16_t* x, uint8_t* codes, float* scales, int tokens, int hidden, hipStream_t stream);
 hipError_t launch_dequantize(const uint8_t* codes, const float* scales, uint16_t* out, int tokens, int hidden, hipStream_t stream);

@@ -915,6 +915,13 @@ int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes,
     return 0;
 }
 
+int pcie_ep_litmus(int32_t device, int32_t mode, int64_t iterations, int32_t payload_bytes, int32_t writer_delay_ns, int32_t reader_delay_ns,
+                   int32_t timeout_ms, pcie_ep_litmus_result* result) {
+    std::string error;
+    const int status = run_litmus(device, mode, iterations, payload_bytes, writer_delay_ns, reader_delay_ns, timeout_ms, result, error);
+    return status ? set_error(status, "%s", error.c_str()) : 0;
+}
+
 // ---- peer emulator -----------------------------------------------------------------
 
 #define NEED_PEERS(rt)                                                                                        \

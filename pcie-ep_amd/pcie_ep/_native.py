@@ -39,6 +39,11 @@ class RelayFlow(C.Structure):
                                         "credit_wait_probes_total", "drained_epoch", "copies_total", "payload_bytes_total")]
 
 
+class LitmusResult(C.Structure):
+    _fields_ = [("completed", C.c_int64), ("gpu_code", C.c_int32), ("host_code", C.c_int32), ("gpu_iteration", C.c_int64),
+                ("gpu_index", C.c_int64), ("host_iteration", C.c_int64), ("host_index", C.c_int64), ("seconds", C.c_double)]
+
+
 class RelaySummary(C.Structure):
     _fields_ = [(name, C.c_int32) for name in ("enabled", "rank", "num_domains", "workers", "flows", "source_page_node")] + [
         ("rank_numa_nodes", C.c_int32 * 16), ("domain_numa_nodes", C.c_int32 * 8), ("domain_bound", C.c_int32 * 8),
@@ -94,6 +99,7 @@ _PROTOTYPES = {
     "pcie_ep_measure_kernel_host_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "pcie_ep_measure_device_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double)]),
     "pcie_ep_measure_row_scatter": (C.c_int, [C.c_int32] * 7 + [C.POINTER(C.c_double)]),
+    "pcie_ep_litmus": (C.c_int, [C.c_int32, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(LitmusResult)]),
     "pcie_ep_peer_set_source": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
     "pcie_ep_peers_start": (C.c_int, [C.c_void_p, C.c_int32, C.c_uint32]),
     "pcie_ep_peers_wait_staged": (C.c_int, [C.c_void_p, C.c_int32]),
