@@ -92,6 +92,22 @@ def test_lopsided_send_receive_ratios():
         check_case(buffer, "fp8-receive-heavy", [4] + [1500] * 7, seed=26, fp8=True)
 
 
+def test_parity_while_other_traffic_saturates_the_link():
+    """Ordering mistakes on the host link only show when it is busy (the hand-off
+    litmus has the numbers): tiny rings, so that every slot, descriptor entry and
+    ACK word is reused dozens of times per dispatch, both wires and both layouts,
+    while kernel-driven copies keep both directions of the link saturated."""
+    from pcie_ep import litmus
+
+    with litmus.link_traffic():
+        with make_buffer(tmax=700, channels=4, hidden=2048, payload_slots=2, descriptor_slots=1) as buffer:
+            for repeat in range(4):
+                check_case(buffer, "busy-link", [700, 650, 1, 700, 0, 333, 700, 700], expand=bool(repeat % 2), seed=40 + repeat)
+        with make_buffer(tmax=300, channels=32, hidden=7168, payload_slots=3, descriptor_slots=2, stage=7, wire_dtype="fp8_e4m3") as buffer:
+            for repeat in range(3):
+                check_case(buffer, "busy-link-fp8", [300] * 8, "multicast" if repeat == 1 else "random", seed=50 + repeat, fp8=True)
+
+
 @pytest.mark.parametrize("rank", [3, 7])
 def test_other_local_rank(rank):
     with make_buffer(rank=rank, channels=3, hidden=512, payload_slots=4, descriptor_slots=4) as buffer:
