@@ -1072,7 +1072,8 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 // the read rate), re-evaluated before every row, so the writes are spread
 // thinly over the whole dispatch whatever the routing's send/receive ratio is.
 // `lead` makes the transmit side end a little earlier than the receive side (by
-// the time the link needs for kTxLeadBytes): a transmitted row is only finished
+// the time the link needs for kTxLeadBytes, at most a quarter of the rows to
+// receive): a transmitted row is only finished
 // when its receivers have acknowledged it, and that round trip then hides
 // behind the last received rows instead of following them.  The rule corrects
 // itself: a direction that falls behind has more left and gets more wavefronts;
@@ -1114,7 +1115,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
                 // wait for the first descriptors.
                 bool prefer_tx = order < kMinTxWaves;
                 if (tx_total >= 0 && rx_total >= 0) {
-                    const int rx_rows = rx_total - rx_head - lead;
+                    const int rx_rows = rx_total - rx_head - (lead < rx_total / 4 ? lead : rx_total / 4);
                     const int64_t tx_left = tx_done ? 0 : kTxWeight * (tx_total - tx_head), rx_left = rx_rows > 0 ? kRxWeight * rx_rows : 0;
                     prefer_tx = rx_done || (tx_left > 0 && 2 * order < waves &&
                                             (order < kMinTxWaves || int64_t(order) * (tx_left + rx_left) < int64_t(waves) * tx_left));
