@@ -56,6 +56,7 @@ class _Ordering:
         self.raw_stream = int(self.stream.cuda_stream)
         self._consumers: Dict[Tuple[int, int], Any] = {}
         self._guard = threading.Lock()
+        self._made_wait: Optional[Tuple[int, int]] = None  # the stream the last dispatch made wait for its result
 
     @staticmethod
     def _key(stream: Any) -> Tuple[int, int]:
@@ -90,8 +91,11 @@ class _Ordering:
             caller_key = (caller.device.index, int(caller.cuda_stream))
             # A producer stream with nothing pending has produced the inputs already:
             # asking is much cheaper than an event record plus a cross-stream wait.
-            if caller_key != own_key and not caller.query():
+            # A stream this buffer has just made wait for a result (synchronous mode)
+            # is busy until that result is there: then the question is skipped too.
+            if caller_key != own_key and (caller_key == self._made_wait or not caller.query()):
                 self.stream.wait_stream(caller)
+            self._made_wait = None
         else:
             caller_key = own_key
             if isinstance(previous_event, EventOverlap):
@@ -259,6 +263,7 @@ class HostStagedEPBuffer:
                    result.get("recv_topk_weights") if request.weights is not None else None, handle)
         if not asynchronous:
             caller.wait_event(done)
+            self._ordering._made_wait = self._ordering._key(caller)
             # The result tensors belong to a pool that was allocated on one stream
             # and lives as long as the buffer; only a consumer on another stream
             # needs to be made known to the caching allocator.
