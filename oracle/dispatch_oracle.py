@@ -19,6 +19,10 @@ Pins (what each function is checked against in ``tests/test_oracle_*.py``):
   invariants (sum of counts, permutation property of rows).
 * ``expand_rows`` / ``unique_rows`` — brute force on tiny inputs and the
   closed form ``argsort(stable)`` of the reference's large test.
+* ``source_statistics`` with a NUMA map (relay descriptors and copies) — an
+  independent per-(token, domain) brute force and the reference's own
+  expectation of one copy per (token, other domain reached)
+  (tests/test_relay.py:16-22); without a map it must equal the deliveries.
 * FP8 functions live in ``fp8_oracle.py`` with their own pins.
 """
 
