@@ -194,7 +194,7 @@ def measure_expand(inputs, tokens, topk, channels, repeats=20):
             ceilings[name] = rate.value
         return {
             "shape_ceiling_GBps": ceilings,
-            "bound": "hbm", "kernel": "expand_kernel", "achieved": algorithmic / mean_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "bound": "hbm", "kernel": "expand_pieces_kernel", "achieved": algorithmic / mean_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": algorithmic / mean_ms / 1e6 / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": algorithmic,
             "avg_us": mean_ms * 1e3, "min_us": min(durations) * 1e3, "unique_rows": unique, "expanded_rows": expanded,
         }
@@ -343,6 +343,40 @@ def graph_replay_sweep(topk, channels, sizes=(16, 128, 512, 2048, 8192), replays
     return out
 
 
+def role_timeline(sizes, wire, channels, repeats=15):
+    """Per-role timeline of the dispatch (profiling build of the library): for every
+    size, `repeats` dispatches submitted one at a time, each read back; the median of
+    every event, in microseconds after the prologue's entry."""
+    import statistics
+
+    import torch
+
+    from pcie_ep import profiling
+
+    out = {}
+    for tokens in sizes:
+        inputs = build_inputs(tokens, 8, "uniform", wire == "fp8")
+        buffer = make_buffer(tokens, 8, wire, channels, fuse=True)
+        try:
+            set_peers(buffer, inputs)
+            x, idx, weights = (item.cuda() for item in inputs[0])
+            buffer.peers.start(5 + repeats)
+            buffer.peers.wait_staged(120_000)
+            samples = []
+            for step in range(5 + repeats):
+                result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+                torch.cuda.synchronize()
+                if step >= 5:
+                    samples.append(profiling.timeline(profiling.read(buffer.runtime)))
+                del result
+            buffer.peers.wait(120_000)
+        finally:
+            buffer.close()
+        out[str(tokens)] = {name: round(statistics.median(sample[name] for sample in samples), 2) for name in samples[0]}
+        log(f"[bench] role timeline T={tokens}: last role exit {out[str(tokens)]['transport.last_role_exit']} us after the prologue's entry")
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
@@ -360,7 +394,12 @@ def main() -> int:
                              "graph-replay / restaged sub-records); what the profiler runs use")
     parser.add_argument("--expand-only", action="store_true",
                         help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
+    parser.add_argument("--role-timeline", type=str, default="",
+                        help="comma-separated token counts: print the per-role timeline of the dispatch at those sizes and exit "
+                             "(needs the profiling build: python pcie-ep_amd/build.py --profiling)")
     args = parser.parse_args()
+    if args.role_timeline:
+        os.environ["PCIE_EP_PROFILING"] = "1"
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the dispatch; --gpus {args.gpus} is not supported "
               "(this build uses no second GPU, no collective and no rank code)", file=sys.stderr)
@@ -371,6 +410,11 @@ def main() -> int:
     from pcie_ep import _native
 
     torch.cuda.set_device(0)
+    if args.role_timeline:
+        sizes = [int(item) for item in args.role_timeline.split(",")]
+        print(json.dumps({"role_timeline_us": role_timeline(sizes, args.wire, args.channels), "wire": args.wire,
+                          "note": "median of 15 dispatches, microseconds after the prologue leader's entry; profiling build"}), flush=True)
+        return 0
     topk = 4 if args.routing == "hotspot" else 8
     tokens = args.tokens
     log(f"[bench] building inputs: T={tokens} H={HIDDEN} top-{topk} {args.routing} {args.wire} wire")

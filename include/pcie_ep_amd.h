@@ -173,6 +173,16 @@ int pcie_ep_dispatch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args
  * (pcie_ep_set_kernel_timing) is not recorded by this entry point. */
 int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
 
+/* Residency of the transport kernel on `compute_units` compute units (0 = the whole
+ * device): `needed` = control + payload workgroups of one dispatch, which wait for
+ * each other through device memory and must therefore all be running at once;
+ * `resident` = workgroups of that kernel the units hold together (occupancy of the
+ * kernel times the units).  A caller that confines the dispatch stream to a
+ * compute-unit mask must keep resident >= needed, otherwise every dispatch ends
+ * with device code 15 after the timeout.  No counterpart in the reference (its
+ * kernels take `num_sms`-style footprints on trust). */
+int pcie_ep_transport_residency(pcie_ep_runtime* runtime, int32_t compute_units, int32_t* needed, int32_t* resident);
+
 /* Thread-local message of the last failing call (runtime may be NULL). */
 const char* pcie_ep_last_error(void);
 
@@ -268,6 +278,20 @@ int pcie_ep_expand_unique(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args*
  * dispatch: benchmarks/benchmark.py:165-198). */
 int pcie_ep_set_kernel_timing(pcie_ep_runtime* runtime, int32_t enable);
 int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds3);
+
+/* Per-role timing records of the last dispatch, from a library built with
+ * -DPCIE_EP_ENABLE_PROFILING=1 (`python pcie-ep_amd/build.py --profiling`; the default
+ * build contains no profiling code and reports 0 rows).  Replaces the `profiling`
+ * output tensor of the reference's PCIE_EP_ENABLE_PROFILING build
+ * (csrc/kernels/host_staged/advanced_common.cuh:126-181; docs/pcie-ep/
+ * profiling-instrumentation.md): one record of `fields` (32) int64 per role wavefront,
+ * rows ordered TX control [0, C), RX control [C, 2C), payload wavefronts
+ * [2C, 2C + W), prologue leader [2C + W]; the field meanings are the ProfileField /
+ * PrologueProfileField enums of csrc/device_common.h, mirrored in pcie_ep/profiling.py.
+ * pcie_ep_profile_read synchronises the device (a diagnostic wait outside the dispatch
+ * path, like the reference's handle.profiling.cpu()). */
+int pcie_ep_profile_shape(pcie_ep_runtime* runtime, int32_t* rows, int32_t* fields, int32_t* channels, int32_t* payload_wavefronts);
+int pcie_ep_profile_read(pcie_ep_runtime* runtime, int64_t* records);
 
 /* Pinned-copy bandwidth of this box (GB/s, best of `repeats`), the denominator
  * for "% of x16 peak".  No counterpart in the reference. */
@@ -365,8 +389,8 @@ int pcie_ep_peer_captured_copy(pcie_ep_runtime* runtime, int32_t rank, int32_t* 
 /* Force a protocol failure from the host.  fault: 1 withhold counts_ready,
  * 2 withhold counts_consumed, 3 withhold the last payload ACK, 4 publish a
  * wrong payload sequence, 5 send a unique-row ordinal beyond the announced
- * count, 6 send an expert ordinal beyond the announced count (4-6 on the last
- * row of every channel).  Applies to rank `rank` for the next started epochs;
+ * count, 6 send an expert ordinal beyond the announced count, 7 name a payload
+ * slot beyond the ring in the descriptor (4-7 on the last row of every channel).  Applies to rank `rank` for the next started epochs;
  * fault 0 clears. */
 int pcie_ep_peers_inject_fault(pcie_ep_runtime* runtime, int32_t rank, int32_t fault);
 

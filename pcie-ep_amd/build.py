@@ -2,6 +2,7 @@
 
     python pcie-ep_amd/build.py            # compile every source, link the .so
     python pcie-ep_amd/build.py --if-missing
+    python pcie-ep_amd/build.py --profiling   # additionally libpcie_ep_amd_profiling.so (per-role timing records)
 
 hipcc cross-compiles for gfx950 without a GPU.  The library lands in
 ``pcie-ep_amd/pcie_ep/lib/libpcie_ep_amd.so`` so it travels with the tree.
@@ -20,6 +21,7 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OUT_DIR = HERE / "pcie_ep" / "lib"
 LIBRARY = OUT_DIR / "libpcie_ep_amd.so"
+PROFILING_LIBRARY = OUT_DIR / "libpcie_ep_amd_profiling.so"
 CLIENT = OUT_DIR / "abi_client"
 OBJ_DIR = HERE / "build"
 
@@ -41,10 +43,12 @@ def _run(command: list[str]) -> None:
         print(stderr, file=sys.stderr)
 
 
-def _compile(name: str) -> Path:
+def _compile(name: str, profiling: bool = False) -> Path:
     source = CSRC / name
-    target = OBJ_DIR / (name + ".o")
+    target = OBJ_DIR / (name + (".profiling.o" if profiling else ".o"))
     command = ["hipcc", *COMMON]
+    if profiling:
+        command.append("-DPCIE_EP_ENABLE_PROFILING=1")
     if name.endswith(".hip"):
         command += DEVICE
     command += ["-c", str(source), "-o", str(target)]
@@ -52,16 +56,29 @@ def _compile(name: str) -> Path:
     return target
 
 
-def build(force: bool = True) -> Path:
-    if not force and LIBRARY.exists():
+def _link(objects: list, library: Path) -> None:
+    _run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-pthread", *map(str, objects), "-o", str(library)])
+
+
+def build(force: bool = True, profiling: bool = False) -> Path:
+    """Compile and link the library; with ``profiling`` also the variant whose
+    kernels keep per-role timing records (same sources, -DPCIE_EP_ENABLE_PROFILING=1)."""
+    if not force and LIBRARY.exists() and (not profiling or PROFILING_LIBRARY.exists()):
         return LIBRARY
     if shutil.which("hipcc") is None:
         raise RuntimeError("hipcc not found: the HIP extension cannot be built")
     OBJ_DIR.mkdir(exist_ok=True)
     OUT_DIR.mkdir(exist_ok=True)
-    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
-        objects = list(pool.map(_compile, HIP_SOURCES + CXX_SOURCES))
-    _run(["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-pthread", *map(str, objects), "-o", str(LIBRARY)])
+    sources = HIP_SOURCES + CXX_SOURCES
+    with concurrent.futures.ThreadPoolExecutor(max_workers=7) as pool:
+        plain = [pool.submit(_compile, name) for name in sources]
+        timed = [pool.submit(_compile, name, True) for name in HIP_SOURCES] if profiling else []
+        objects = [job.result() for job in plain]
+        timed_objects = [job.result() for job in timed]
+    _link(objects, LIBRARY)
+    if profiling:
+        # The host-only sources do not depend on the switch.
+        _link(timed_objects + objects[len(HIP_SOURCES):], PROFILING_LIBRARY)
     build_client()
     return LIBRARY
 
@@ -79,5 +96,6 @@ def build_client() -> Path:
 if __name__ == "__main__":
     parser = argparse.ArgumentParser()
     parser.add_argument("--if-missing", action="store_true")
+    parser.add_argument("--profiling", action="store_true")
     arguments = parser.parse_args()
-    print(build(force=not arguments.if_missing))
+    print(build(force=not arguments.if_missing, profiling=arguments.profiling))

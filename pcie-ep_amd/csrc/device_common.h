@@ -10,6 +10,22 @@
 namespace pcie_ep {
 
 constexpr int kWave = 64;
+
+// Per-role timing records, compiled in only with -DPCIE_EP_ENABLE_PROFILING=1 (the
+// reference's switch of the same name: csrc/kernels/host_staged/advanced_common.cuh:
+// 126-181, docs/pcie-ep/profiling-instrumentation.md).  A default build contains
+// none of it: the macro below expands to nothing and DeviceState has no field for it.
+#ifndef PCIE_EP_ENABLE_PROFILING
+#define PCIE_EP_ENABLE_PROFILING 0
+#endif
+#if PCIE_EP_ENABLE_PROFILING
+#define PCIE_EP_PROFILE(...) __VA_ARGS__
+#else
+#define PCIE_EP_PROFILE(...)
+#endif
+constexpr int kProfileFields = 32;
+constexpr int kProfileSampleStride = 8;  // every 8th row of a payload wavefront is timed in detail
+
 constexpr uint64_t kPrefixFailed = ~uint64_t(0);
 // Set in the claim word of the receive prefixes once their producer has put its
 // reads of the count mailboxes on the host link.
@@ -136,6 +152,10 @@ struct DeviceState {
     uint64_t* receive_prefix_state;
     int64_t* prefix_tx_timestamps_ns;
 
+#if PCIE_EP_ENABLE_PROFILING
+    int64_t* profiling;  // [profile_rows(...)][kProfileFields], one row per role wavefront (profiling builds only)
+#endif
+
     // Test hooks, in clock ticks (advanced_common.cuh:118-124).
     uint64_t metadata_delay;
     uint64_t tx_delay;
@@ -154,6 +174,74 @@ __device__ __forceinline__ int64_t ticks_to_ns(const DeviceState& state, uint64_
     return int64_t(ticks / khz * 1000000ull + ticks % khz * 1000000ull / khz);
 }
 __device__ __forceinline__ void backoff() { __builtin_amdgcn_s_sleep(8); }
+
+#if PCIE_EP_ENABLE_PROFILING
+// Fields of one role's record.  Times are nanoseconds of the device's wall clock
+// (absolute stamps end in Ns, accumulated intervals in Sum); a zero stamp means
+// the event did not happen.  Each record has one writer (lane 0 of the role's
+// wavefront), is kept in registers and written once when the role ends: no reset
+// kernel, fence, barrier or atomic is added (as in the reference).  Intervals of
+// different roles overlap and must not be added up.
+enum ProfileField : int {
+    kProfileEnterNs = 0, kProfileExitNs, kProfileTotalNs, kProfileItems,
+    // ---- control wavefronts (rows [0, 2C)) ----
+    kProfileFirstTicketNs = 4,   // TX control: first ticket handed out; RX control: first descriptor accepted
+    kProfileLastTicketNs,        // ... and the last one
+    kProfileWorkersDoneNs,       // TX control: all own rows written and published; RX control: all rows scattered
+    kProfileDrainedNs,           // TX control: last payload ACK seen
+    kProfileFinishedNs,          // both directions of the channel complete (TX control) / rx_finished stored (RX control)
+    kProfilePolls,               // TX control: ACK drain passes; RX control: descriptor polls
+    kProfilePollMisses,          // ... that found nothing new
+    kProfilePollSum,             // time inside those polls
+    kProfileHealthScans, kProfileHealthSum,
+    kProfileCountsKnownNs,       // RX control: receive prefixes seen
+    kProfileGateOpenNs,          // RX control: first ticket allowed out (count mailbox reads are on the link)
+    // receive-prefix producer (in the record of the RX control that was elected)
+    kProfilePrefixEnterNs = 16, kProfilePrefixCountsReadyNs, kProfilePrefixMailboxNs, kProfilePrefixPublishedNs,
+    // ---- payload wavefronts (rows [2C, 2C + W)); field 3 = rows moved ----
+    kProfileFirstClaimNs = 4,
+    kProfileLastRowNs,           // end of this wavefront's last row
+    kProfileTxRows, kProfileRxRows,
+    kProfileSampledTxRows, kProfileSampledRxRows,  // rows timed in detail (every kProfileSampleStride-th)
+    kProfileTicketWaitSum,       // claim -> ticket marked ready (all rows)
+    kProfileIdleSum,             // time with nothing to claim
+    kProfileTxFlowWaitSum,       // sampled: slot ACK / descriptor credit wait
+    kProfileTxCopySum,           // sampled: row + metadata stores issued -> acknowledged by the host
+    kProfileRxRequestSum,        // sampled: row loads issued -> metadata and payload returned
+    kProfileRxPrefixWaitSum,     // sampled: waiting for the receive prefixes (first rows only)
+    kProfileRxScatterSum,        // sampled: row loads issued -> destination rows' stores issued
+};
+// Record of the prologue's leader workgroup (thread 0), stored behind the payload wavefronts' records.
+enum PrologueProfileField : int {
+    kPrologueLayoutNs = 4,     // own chunk's ordinals written
+    kPrologueTotalsNs,         // totals of all chunks summed
+    kPrologueVerdictNs,        // abort words and counts_consumed (host loads issued at entry) looked at
+    kPrologueMailboxFreeNs,    // previous count mailbox seen consumed by every peer
+    kPrologueMailboxAckedNs,   // count mailbox stores acknowledged by the host
+    kPrologueCountsReadyNs,    // counts_ready stored
+};
+// Rows of the table: TX controls [0, C), RX controls [C, 2C), payload wavefronts, prologue leader.
+__host__ __device__ inline int profile_rows(int channels, int payload_wavefronts) { return 2 * channels + payload_wavefronts + 1; }
+struct RoleProfile {
+    uint64_t values[kProfileFields] = {};
+    uint64_t khz;
+    __device__ explicit RoleProfile(uint64_t clock_khz) : khz(clock_khz) { values[kProfileEnterNs] = now(); }
+    __device__ __forceinline__ uint64_t now() const {
+        const uint64_t ticks = wall_clock64();
+        asm volatile("" ::: "memory");
+        return ticks / khz * 1000000ull + ticks % khz * 1000000ull / khz;
+    }
+    __device__ __forceinline__ void first(int field) { if (!values[field]) values[field] = now(); }
+    __device__ __forceinline__ void last(int field) { values[field] = now(); }
+    __device__ __forceinline__ void add(int field, uint64_t amount = 1) { values[field] += amount; }
+    __device__ void save(int64_t* table, int row, int lane) {
+        values[kProfileExitNs] = now();
+        values[kProfileTotalNs] = values[kProfileExitNs] - values[kProfileEnterNs];
+        if (lane == 0 && table)
+            for (int field = 0; field < kProfileFields; ++field) table[size_t(row) * kProfileFields + field] = int64_t(values[field]);
+    }
+};
+#endif
 
 __device__ inline void test_delay(uint64_t ticks) {
     if (!ticks) return;
@@ -300,6 +388,17 @@ __device__ __forceinline__ uint32_t device_load_b32(__amdgpu_buffer_rsrc_t resou
 }
 __device__ __forceinline__ void device_store_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint32_t value) {
     __builtin_amdgcn_raw_buffer_store_b32(value, resource, int(byte_offset), 0, kDevicePolicy);
+}
+
+// Streaming row accesses in device memory: buffer instructions with the non-temporal
+// policy.  Lanes beyond the resource's size read zero / are dropped, so rows need no
+// per-lane predicate, and the instruction stream of a row is branch-free.
+constexpr int kStreamPolicy = 2;  // nt
+__device__ __forceinline__ u32x4 stream_load_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset) {
+    return __builtin_amdgcn_raw_buffer_load_b128(resource, int(byte_offset), 0, kStreamPolicy);
+}
+__device__ __forceinline__ void stream_store_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, u32x4 value) {
+    __builtin_amdgcn_raw_buffer_store_b128(value, resource, int(byte_offset), 0, kStreamPolicy);
 }
 
 // ---- device-scope flags in HBM -----------------------------------------------

@@ -55,6 +55,8 @@ size_t prologue_scratch_bytes(const SegmentLayout& z);
 // alignment-gap zeroing and the statistics reduction.
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream);
 int transport_threads(const DeviceState& state);
+// Transport workgroups (of the instantiation `state` selects) that one compute unit holds at once.
+hipError_t transport_workgroups_per_unit(const DeviceState& state, int* per_unit);
 // Stand-alone expand of unique rows into expert-major rows (+ padding).
 hipError_t launch_expand(const DeviceState& state, hipStream_t stream);
 // Plain device-to-device copy of `bytes` (multiple of 16) with the row movers' access shape.

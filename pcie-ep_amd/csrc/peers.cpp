@@ -8,6 +8,10 @@
 
 #include "fp8.h"
 
+#if defined(__x86_64__)
+#include <emmintrin.h>
+#endif
+
 namespace pcie_ep {
 
 namespace {
@@ -17,6 +21,26 @@ inline void release(uint64_t* address, uint64_t value) { std::atomic_ref<uint64_
 inline double now_seconds() {
     return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
+// Staging copy of an emulated source.  A real peer is another GPU whose rows reach
+// this memory as DMA writes: they land in memory (or the shared last-level cache),
+// never in a core's private cache.  A plain memcpy would leave the rows modified in
+// the staging core's cache, and every read of the receiving GPU would first have to
+// be snooped out of that core - the emulator would then decide how fast small
+// dispatches run.  Streaming (non-temporal) stores put the rows where a device
+// would, and the fence orders them before the descriptor's release store.
+inline void stage_bytes(char* destination, const void* source, size_t bytes) {
+#if defined(__x86_64__)
+    if (reinterpret_cast<uintptr_t>(destination) % 16 == 0 && bytes % 16 == 0) {
+        const char* from = static_cast<const char*>(source);
+        for (size_t at = 0; at < bytes; at += 16)
+            _mm_stream_si128(reinterpret_cast<__m128i*>(destination + at), _mm_loadu_si128(reinterpret_cast<const __m128i*>(from + at)));
+        _mm_sfence();
+        return;
+    }
+#endif
+    std::memcpy(destination, source, bytes);
+}
+
 inline void cpu_relax() {
 #if defined(__x86_64__)
     __builtin_ia32_pause();
@@ -190,7 +214,7 @@ void PeerEmulator::cancel() {
 }
 
 int PeerEmulator::inject_fault(int rank, int fault) {
-    if (rank < 0 || rank >= z_.dims.num_ranks || rank == me_ || fault < 0 || fault > kFaultExpertOrdinalOutOfRange) return -1;
+    if (rank < 0 || rank >= z_.dims.num_ranks || rank == me_ || fault < 0 || fault > kFaultSlotOutOfRange) return -1;
     ranks_[rank].fault.store(fault);
     return 0;
 }
@@ -326,10 +350,17 @@ void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int chan
     if ((flags_ & kPeerRestage) || falsify || state.slot_generation[slot_index] != state.generation || state.slot_token[slot_index] != token) {
         float scale = 1.0f;
         const uint16_t* row = state.x.data() + size_t(token) * hidden;
-        if (z_.dims.wire_fp8) host_quantize_fp8(row, reinterpret_cast<uint8_t*>(base), &scale, 1, hidden);
-        else std::memcpy(base, row, size_t(hidden) * 2);
-        char* meta = base + z_.meta_offset;
-        std::memset(meta, 0, z_.meta_bytes);
+        if (z_.dims.wire_fp8) {
+            std::vector<uint8_t>& codes = state.stage_codes;
+            codes.resize((size_t(hidden) + 15) / 16 * 16);
+            host_quantize_fp8(row, codes.data(), &scale, 1, hidden);
+            if (hidden % 16 == 0) stage_bytes(base, codes.data(), size_t(hidden));
+            else std::memcpy(base, codes.data(), size_t(hidden));
+        } else {
+            stage_bytes(base, row, size_t(hidden) * 2);
+        }
+        // The slot metadata is composed on the side and staged the same way.
+        alignas(16) char meta[kMetaBranchOffset + 12 * kMaxTopk + 16] = {};
         SlotMetaHeader header{};
         header.token_index = token;
         header.destination_mask = state.mask[token];
@@ -351,9 +382,10 @@ void PeerEmulator::publish_token(Rank& state, int rank, uint64_t epoch, int chan
                     if (branch[k] >= 0 && branch[k] / z_.local_experts == me_) branch[topk + k] = 1 << 20;
             state.slot_token[slot_index] = -1;  // stage the true row again next time
         }
+        stage_bytes(base + z_.meta_offset, meta, size_t(z_.meta_bytes));
     }
     Descriptor* descriptor = descriptor_at(z_, own, channel, endpoint_of(z_.dims, rank, me_), ordinal);
-    descriptor->payload_slot = slot;
+    descriptor->payload_slot = fault == kFaultSlotOutOfRange ? z_.dims.payload_slots : slot;
     // The token identifies the payload (its sequence is sequence(epoch, token));
     // the fault hook publishes a token that does not match the slot's metadata.
     descriptor->token_index = fault == kFaultWrongPayloadSequence ? token + 1 : token;

@@ -37,6 +37,7 @@ enum PeerFault : int {
     kFaultWrongPayloadSequence = 4,
     kFaultRankOrdinalOutOfRange = 5,    // last row: unique-row ordinal beyond the announced count
     kFaultExpertOrdinalOutOfRange = 6,  // last row: expert ordinal beyond the announced count
+    kFaultSlotOutOfRange = 7,           // last row: the descriptor names a payload slot beyond the ring
 };
 
 // Flags of PeerEmulator::start.
@@ -97,6 +98,7 @@ private:
         std::vector<uint32_t> cap_masks;
         std::atomic<int> fault{0};
         uint64_t read_checksum = 0;  // sink of kPeerReadRows
+        std::vector<uint8_t> stage_codes;  // FP8 codes of the row being staged
         std::atomic<uint64_t> staged_epoch{0};
     };
 

@@ -28,7 +28,7 @@ namespace pcie_ep {
 
 namespace {
 
-__device__ void publish_counts(const DeviceState& state, uint64_t epoch) {
+__device__ void publish_counts(const DeviceState& state, uint64_t epoch PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const SegmentLayout& z = state.z;
     char* own = state.seg[state.local_rank];
     const int ranks = z.dims.num_ranks, local = z.local_experts;
@@ -52,7 +52,9 @@ __device__ void publish_counts(const DeviceState& state, uint64_t epoch) {
     // (a leader-only wait would not cover the other writers: layout.cuh:21-28).
     wait_memory_ops();
     __syncthreads();
+    PCIE_EP_PROFILE(profile.first(kPrologueMailboxAckedNs);)
     if (threadIdx.x == 0) host_store_release(signal_at(own, z.counts_ready_offset), epoch);
+    PCIE_EP_PROFILE(profile.first(kPrologueCountsReadyNs);)
 }
 
 }  // namespace
@@ -87,6 +89,8 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     // so every workgroup of the launch reads the same (previous) epoch here.
     const uint64_t tag = *state.epoch + 1;
     const uint64_t begin_ticks = now_ticks();
+    PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);
+                    const int profile_row = profile_rows(channels, (state.worker_groups > 0 ? state.worker_groups : channels) * (state.tx_waves + state.rx_waves)) - 1;)
     __shared__ int stalled;
     if (threadIdx.x == 0) stalled = 0;
 
@@ -259,6 +263,7 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         }
     }
     if (!leader) return;
+    PCIE_EP_PROFILE(profile.first(kPrologueLayoutNs);)
 
     // ---- leader: totals of the whole plan ------------------------------------------------
     if (!state.reuse_plan) {
@@ -293,6 +298,7 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         }
     }
 
+    PCIE_EP_PROFILE(profile.first(kPrologueTotalsNs);)
     // ---- epoch verdict -----------------------------------------------------------------
     // Everything the leader's threads hand to each other below (plan totals, the
     // error record) stays inside this workgroup: the barriers order it, no cache
@@ -302,6 +308,7 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     for (int i = 0; i < kAbortLoadsPerThread; ++i) aborted |= abort_words[i] != 0;
     bool consumed = consumed_word == tag - 1;
     const bool any_abort = __syncthreads_or(aborted);
+    PCIE_EP_PROFILE(profile.first(kPrologueVerdictNs);)
     if (threadIdx.x == 0) {
         *state.epoch = tag;
         if (tag >= 0x100000000ull) record_error(state, kErrEpochExhausted);
@@ -315,7 +322,10 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
     __shared__ int mailbox_failed;
     if (threadIdx.x == 0) mailbox_failed = 0;
     __syncthreads();
-    if (load_error_code(state)) return;
+    if (load_error_code(state)) {
+        PCIE_EP_PROFILE(profile.save(state.profiling, profile_row, threadIdx.x);)
+        return;
+    }
 
     // ---- previous count mailbox must be consumed by every peer --------------------------
     // (advanced_layout.cuh:60-88): only then may the counts be overwritten.
@@ -335,14 +345,19 @@ __global__ void __launch_bounds__(kPrologueMaxThreads) prologue_kernel(DeviceSta
         }
     }
     __syncthreads();
-    if (mailbox_failed) return;
+    PCIE_EP_PROFILE(profile.first(kPrologueMailboxFreeNs);)
+    if (mailbox_failed) {
+        PCIE_EP_PROFILE(profile.save(state.profiling, profile_row, threadIdx.x);)
+        return;
+    }
     // Transmit tickets of this dispatch: every own token with a remote destination.
     if (threadIdx.x == 0) {
         int remote_tokens = 0;
         for (int channel = 0; channel < channels; ++channel) remote_tokens += state.plan_chan_remote[channel];
         state.queues->tx_head.total = remote_tokens;
     }
-    publish_counts(state, epoch);
+    publish_counts(state, epoch PCIE_EP_PROFILE(, profile));
+    PCIE_EP_PROFILE(profile.save(state.profiling, profile_row, threadIdx.x);)
 }
 
 size_t prologue_lds_bytes(const SegmentLayout& z, int chunk_waves) {

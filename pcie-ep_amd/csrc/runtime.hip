@@ -31,6 +31,8 @@
 
 using namespace pcie_ep;
 
+struct pcie_ep_runtime;
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -168,6 +170,9 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 std::mutex g_scratch_guard;
 unsigned char* g_scratch_address[kStaticScratchDevices] = {};
+// The runtime whose dispatch used this GPU's array last; its `scratch_done` event
+// says whether that dispatch has finished.
+pcie_ep_runtime* g_scratch_user[kStaticScratchDevices] = {};
 
 // Device address of `scratch` on `device`, which must be the current device.
 int static_scratch_of(int device, unsigned char** address) {
@@ -254,6 +259,12 @@ struct pcie_ep_runtime {
     bool timing_valid = false;
     bool timing_expand = false;
     hipEvent_t marks[4] = {};
+    // Recorded behind every dispatch through the static scratch (created with the runtime:
+    // that entry point must not allocate).
+    hipEvent_t scratch_done = nullptr;
+    // Profiling builds: [profile_rows][kProfileFields] records in device memory.
+    int64_t* profiling = nullptr;
+    int profile_row_count = 0;
 };
 
 namespace {
@@ -366,6 +377,9 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.receive_expand_overlap = a->receive_expand_overlap;
     s.receive_prefix_state = a->receive_prefix_state;
     s.prefix_tx_timestamps_ns = a->prefix_tx_timestamps_ns;
+#if PCIE_EP_ENABLE_PROFILING
+    s.profiling = rt->profiling;
+#endif
     s.metadata_delay = rt->metadata_delay;
     s.tx_delay = rt->tx_delay;
     s.rx_delay = rt->rx_delay;
@@ -469,6 +483,13 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (error == hipSuccess) error = hipMemset(rt->queues, 0, sizeof(TransportQueues));
         if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->layout_scratch), prologue_scratch_bytes(rt->z));
         if (error == hipSuccess) error = hipMemset(rt->layout_scratch, 0, prologue_scratch_bytes(rt->z));
+        if (error == hipSuccess) error = hipEventCreateWithFlags(&rt->scratch_done, hipEventDisableTiming);
+#if PCIE_EP_ENABLE_PROFILING
+        rt->profile_row_count = profile_rows(dims.channels, (rt->worker_groups > 0 ? rt->worker_groups : dims.channels) * (rt->tx_waves + rt->rx_waves));
+        const size_t profile_bytes = size_t(rt->profile_row_count) * kProfileFields * sizeof(int64_t);
+        if (error == hipSuccess) error = hipMalloc(reinterpret_cast<void**>(&rt->profiling), profile_bytes);
+        if (error == hipSuccess) error = hipMemset(rt->profiling, 0, profile_bytes);
+#endif
         if (error == hipSuccess) error = hipDeviceSynchronize();
         if (error != hipSuccess) status = set_error(PCIE_EP_E_HIP, "device workspace allocation failed: %s", hipGetErrorString(error));
     }
@@ -481,6 +502,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
         if (rt->queues) (void)hipFree(rt->queues);
         if (rt->layout_scratch) (void)hipFree(rt->layout_scratch);
+        if (rt->scratch_done) (void)hipEventDestroy(rt->scratch_done);
+        if (rt->profiling) (void)hipFree(rt->profiling);
         return status;
     }
     RelayOptions relay_options;
@@ -523,6 +546,13 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     if (rt->layout_scratch) (void)hipFree(rt->layout_scratch);
     for (hipEvent_t mark : rt->marks)
         if (mark) (void)hipEventDestroy(mark);
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_guard);
+        for (pcie_ep_runtime*& user : g_scratch_user)
+            if (user == rt) user = nullptr;
+    }
+    if (rt->scratch_done) (void)hipEventDestroy(rt->scratch_done);
+    if (rt->profiling) (void)hipFree(rt->profiling);
     delete rt;
     return status;
 }
@@ -568,12 +598,29 @@ int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* rt, const pcie_ep_dispatch_
     // here they point into this GPU's static array instead of the runtime's own
     // allocations.  Only the epoch counter, which is state of the host rings and
     // not scratch, stays where pcie_ep_runtime_create put it.
+    hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+    // Every runtime on this GPU shares the one array.  A dispatch of ANOTHER runtime
+    // that has not finished yet would have its ticket queues cleared under it: refuse
+    // instead.  (Calls of one runtime are ordered by its caller anyway.)  Under stream
+    // capture nothing executes now and an event cannot be queried: the check is
+    // skipped there, and replays of such a graph are the caller's to order.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(stream, &capture));
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> scratch_lock(g_scratch_guard);
+    if (!capturing) {
+        pcie_ep_runtime* last = g_scratch_user[rt->config.device];
+        if (last && last != rt && hipEventQuery(last->scratch_done) == hipErrorNotReady)
+            return set_error(PCIE_EP_E_STATE, "the static scratch of device %d is in use by a dispatch of another runtime that has not finished",
+                             rt->config.device);
+    }
+    // Per-kernel timing is not recorded here; stamps of an earlier ordinary dispatch must not pass for this one's.
+    rt->timing_valid = false;
     unsigned char* base = rt->static_scratch;
     state.queues = reinterpret_cast<TransportQueues*>(base + carve.queues);
     state.layout_flags = reinterpret_cast<uint64_t*>(base + carve.layout);
     state.layout_records = reinterpret_cast<int32_t*>(base + carve.layout + prologue_flag_bytes(rt->z));
     state.chan_remote_tokens = reinterpret_cast<int32_t*>(base + carve.history);
-    hipStream_t stream = static_cast<hipStream_t>(stream_handle);
     // The array keeps what its last user left, possibly another runtime whose
     // epoch numbers coincide with this one's: the epoch-tagged words (ticket ring
     // tags, queue counters, prologue chunk flags) start from zero.  A fill kernel,
@@ -582,6 +629,49 @@ int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* rt, const pcie_ep_dispatch_
     HIP_TRY(launch_prologue(state, stream));
     HIP_TRY(launch_transport(state, stream));
     if (state.expand && !state.fuse_expand) HIP_TRY(launch_expand(state, stream));
+    if (!capturing) {
+        HIP_TRY(hipEventRecord(rt->scratch_done, stream));
+        g_scratch_user[rt->config.device] = rt;
+    }
+    return 0;
+}
+
+int pcie_ep_transport_residency(pcie_ep_runtime* rt, int32_t compute_units, int32_t* needed, int32_t* resident) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!needed || !resident || compute_units < 0) return set_error(PCIE_EP_E_INVALID, "bad residency arguments");
+    HIP_TRY(hipSetDevice(rt->config.device));
+    int units = compute_units;
+    if (!units) HIP_TRY(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, rt->config.device));
+    DeviceState probe{};
+    probe.z = rt->z;
+    probe.tx_waves = rt->tx_waves;
+    probe.rx_waves = rt->rx_waves;
+    probe.worker_groups = rt->worker_groups;
+    int per_unit = 0;
+    HIP_TRY(transport_workgroups_per_unit(probe, &per_unit));
+    // The control and payload workgroups wait for each other through device memory
+    // and must run together; the local-bypass workgroups behind them may start late.
+    *needed = rt->z.dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0);
+    *resident = per_unit * units;
+    return 0;
+}
+
+int pcie_ep_profile_shape(pcie_ep_runtime* rt, int32_t* rows, int32_t* fields, int32_t* channels, int32_t* payload_wavefronts) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!rows || !fields || !channels || !payload_wavefronts) return set_error(PCIE_EP_E_INVALID, "bad profile arguments");
+    *rows = rt->profile_row_count;  // 0: the library was built without PCIE_EP_ENABLE_PROFILING
+    *fields = kProfileFields;
+    *channels = rt->z.dims.channels;
+    *payload_wavefronts = (rt->worker_groups > 0 ? rt->worker_groups : rt->z.dims.channels) * (rt->tx_waves + rt->rx_waves);
+    return 0;
+}
+
+int pcie_ep_profile_read(pcie_ep_runtime* rt, int64_t* records) {
+    if (!rt || rt->closed) return set_error(PCIE_EP_E_STATE, "advanced runtime is closed or closing");
+    if (!rt->profiling) return set_error(PCIE_EP_E_STATE, "this library was built without PCIE_EP_ENABLE_PROFILING");
+    if (!records) return set_error(PCIE_EP_E_INVALID, "bad profile arguments");
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(records, rt->profiling, size_t(rt->profile_row_count) * kProfileFields * sizeof(int64_t), hipMemcpyDeviceToHost));
     return 0;
 }
 

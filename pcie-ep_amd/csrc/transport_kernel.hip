@@ -122,13 +122,14 @@ __device__ inline int wait_ticket(const DeviceState& state, TransportQueues& q, 
 // elected by a device-scope CAS; it waits for every source's counts_ready,
 // folds the mailboxes in rank order and publishes a generation-valued READY.
 // ---------------------------------------------------------------------------------------
-__device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
+__device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, local = z.local_experts, channels = z.dims.channels;
     const int me = state.local_rank;
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
     HealthCheck health(state, start);
+    PCIE_EP_PROFILE(profile.first(kProfilePrefixEnterNs);)
     if (lane == 0) {
         state.prefix_tx_timestamps_ns[0] = ticks_to_ns(state, start);
         test_delay(state.prefix_delay);
@@ -186,6 +187,7 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     }
     wait_memory_ops();
     compiler_barrier();
+    PCIE_EP_PROFILE(profile.first(kProfilePrefixCountsReadyNs);)
     int unique = 0;
     if (unique_address) unique = host_field_load_global(unique_address);
     int expected_values[kExpectedPerLane];
@@ -201,6 +203,7 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane) {
     compiler_barrier();
     // Per-source unique counts -> source_offsets (lane = source).
     int inclusive = unique;
+    PCIE_EP_PROFILE(if (__builtin_amdgcn_readfirstlane(inclusive) >= 0) profile.first(kProfilePrefixMailboxNs);)  // the first use of a mailbox word: the reads have returned
     for (int offset = 1; offset < kMaxRanks; offset <<= 1) {
         const int other = __shfl_up(inclusive, offset);
         if (lane >= offset) inclusive += other;
@@ -271,7 +274,7 @@ __device__ void acknowledge_counts(const DeviceState& state, int lane) {
 
 // One wavefront of the grid (the first RX control to get there) computes the
 // receive prefixes; nobody waits here.
-__device__ void elect_receive_prefixes(const DeviceState& state, int lane) {
+__device__ void elect_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const uint64_t epoch = *state.epoch;
     int claimed = 0;
     if (lane == 0) {
@@ -279,7 +282,7 @@ __device__ void elect_receive_prefixes(const DeviceState& state, int lane) {
         claimed = atomicCAS(reinterpret_cast<unsigned long long*>(state.receive_prefix_state), expected, epoch) == 0ull;
     }
     if (!broadcast_first(claimed)) return;
-    const bool success = compute_receive_prefixes(state, lane);
+    const bool success = compute_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
     // The results were written through; they are complete once this wavefront's
     // stores have been acknowledged.  Local consumers come first, the ACK to the
     // sources (which nobody on this GPU waits for) second.
@@ -288,6 +291,7 @@ __device__ void elect_receive_prefixes(const DeviceState& state, int lane) {
         state.prefix_tx_timestamps_ns[1] = ticks_to_ns(state, now_ticks());
         device_store(state.receive_prefix_state + 1, success ? epoch : kPrefixFailed);
     }
+    PCIE_EP_PROFILE(profile.first(kProfilePrefixPublishedNs);)
     if (success) acknowledge_counts(state, lane);
 }
 
@@ -318,6 +322,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     const uint64_t epoch = *state.epoch;
     const uint64_t start = now_ticks();
     HealthCheck health(state, start, true, channel, channels);
+    PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
     if (lane == 0) device_store(state.channel_timestamps_ns + channel * 2, ticks_to_ns(state, start));
     const int tokens = state.num_tokens;
     const int candidates = tokens > channel ? (tokens - channel + channels - 1) / channels : 0;
@@ -388,7 +393,9 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
             backoff();
         }
         produced += __popcll(batch);
+        PCIE_EP_PROFILE(profile.first(kProfileFirstTicketNs); profile.last(kProfileLastTicketNs);)
     }
+    PCIE_EP_PROFILE(profile.values[kProfileItems] = uint64_t(produced);)
 
     // Wait for the workers, then drain the ACKs of the last ring window: earlier
     // slots were checked when they were reused (advanced_dispatch.cuh:229-285).
@@ -403,7 +410,10 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     bool workers_finished = false;
     while (true) {
         if (broadcast_first(aborted(q) ? 1 : 0)) break;
-        if (!workers_finished) workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
+        if (!workers_finished) {
+            workers_finished = broadcast_first(int(device_load(&q.tx_retired[channel].value))) >= produced;
+            PCIE_EP_PROFILE(if (workers_finished) profile.first(kProfileWorkersDoneNs);)
+        }
         if (workers_finished && !drained) {
             // Each pass checks up to kDrainBatch * (64 / endpoints) ordinals of every
             // endpoint; lanes of one endpoint read consecutive ACK words (one 64-byte read
@@ -414,6 +424,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
             // compete with the row reads for the link.
             const bool receive_busy = broadcast_first(int(device_load(&q.rx_finished[channel].value))) == 0;
             if (!receive_busy || broadcast_first(now_ticks() >= next_drain_poll ? 1 : 0)) {
+                PCIE_EP_PROFILE(const uint64_t poll_begin = profile.now(); profile.add(kProfilePolls);)
                 constexpr int kDrainBatch = 8;
                 const int group = kWave / endpoints;
                 const int per_pass = group * kDrainBatch;
@@ -453,6 +464,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
                 drain_ordinal = missing_ordinal < drain_ordinal + per_pass ? missing_ordinal : drain_ordinal + per_pass;
                 if (drain_ordinal >= produced) drained = true;
                 else if (missing_ordinal != 0x7FFFFFFF) next_drain_poll = now_ticks() + 20 * state.clock_khz / 1000;
+                PCIE_EP_PROFILE(profile.add(kProfilePollSum, profile.now() - poll_begin); if (drained) profile.first(kProfileDrainedNs); else profile.add(kProfilePollMisses);)
             }
         }
         if (workers_finished && drained && !relays_drained) {
@@ -462,7 +474,9 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         }
         if (workers_finished && drained && (relays_drained || failed) && broadcast_first(int(device_load(&q.rx_finished[channel].value)))) break;
         // Guardian: this wavefront outlives TX so that a stalled RX still times out.
+        PCIE_EP_PROFILE(const uint64_t health_begin = profile.now();)
         const bool unhealthy = health.poll(state, lane);
+        PCIE_EP_PROFILE(profile.add(kProfileHealthSum, profile.now() - health_begin);)
         const bool forced = channel == 0 && state.control_abort_after && now_ticks() - start >= state.control_abort_after;
         if (unhealthy || broadcast_first(forced ? 1 : 0)) {
             if (lane == 0) {
@@ -483,6 +497,8 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
         // Both directions are complete (or aborted): the channel's end time.
         device_store(state.channel_timestamps_ns + channel * 2 + 1, ticks_to_ns(state, now_ticks()));
     }
+    PCIE_EP_PROFILE(profile.values[kProfileHealthScans] = uint64_t(health.scans); if (produced == 0) profile.first(kProfileDrainedNs);
+                    profile.last(kProfileFinishedNs); profile.save(state.profiling, channel, lane);)
 }
 
 // ---------------------------------------------------------------------------------------
@@ -493,7 +509,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
     const int ranks = z.dims.num_ranks, me = state.local_rank;
     const uint64_t begin = now_ticks();
     const uint64_t epoch = *state.epoch;
-    elect_receive_prefixes(state, lane);
+    PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
+    elect_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
     // Polling does not wait for the prefixes: a descriptor entry is valid as soon as
     // its tag carries this epoch and the next ordinal, whatever the counts say, so
     // rows are requested from the first microseconds of the kernel on.  The counts
@@ -527,6 +544,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                 total = ahead == 0 ? expected : 0;
                 for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset);
                 counts_known = true;
+                PCIE_EP_PROFILE(profile.first(kProfileCountsKnownNs);)
             }
         }
         if (counts_known && issued >= total) break;
@@ -539,7 +557,9 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                                          : descriptor_at(z, segment, channel, me, want ? ordinal : 0);
         // One 16-byte load brings READY together with the slot and token it guards.
         u32x4 published = {0u, 0u, 0u, 0u};
+        PCIE_EP_PROFILE(const uint64_t poll_begin = profile.now(); profile.add(kProfilePolls);)
         if (want) published = host_load_b128_at(descriptor);
+        PCIE_EP_PROFILE(profile.add(kProfilePollSum, profile.now() - poll_begin);)
         const bool ready = want && (uint64_t(published[0]) | uint64_t(published[1]) << 32) == sequence(epoch, ordinal);
         const uint64_t ready_lanes = __ballot(ready);
         // Descriptors of one source are consumed in order: accept the leading run.
@@ -548,9 +568,27 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         const bool accept = ready && ahead < run;
         const uint64_t accepted = __ballot(accept);
         if (!accepted) {
+            PCIE_EP_PROFILE(profile.add(kProfilePollMisses);)
             ++not_ready;
             backoff();
             continue;
+        }
+        // Slot and token come from the peer (or its relay) and become the base of a
+        // host read: a value outside the ring would make the payload wavefront read
+        // beyond the pinned segment, which is a memory fault, not a protocol error.
+        // Same verdict as a wrong identity: terminal, nothing is ACKed.
+        {
+            const int named_slot = int(published[2]), named_token = int(published[3]);
+            const int ring_slots = replica ? z.dims.replica_slots : z.dims.payload_slots;
+            const bool outside = accept && (named_slot < 0 || named_slot >= ring_slots || named_token < 0 || named_token >= z.dims.max_tokens);
+            if (__any(outside)) {
+                if (lane == 0) {
+                    record_error(state, kErrPayloadSequence);
+                    raise_abort(q);
+                }
+                failed = true;
+                break;
+            }
         }
         // The descriptors are polled from the start (a few dozen bytes per source),
         // but no row is handed out before the producer of the prefixes has requested
@@ -567,6 +605,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             } else backoff();
         }
         if (prefix_failed) break;
+        PCIE_EP_PROFILE(profile.first(kProfileGateOpenNs);)
         const int ticket_index = reserve_tickets(q.rx_tail, __popcll(accepted), lane) + __popcll(accepted & below);
         const int slot = int(published[2]), token = int(published[3]);
         const uint64_t payload_sequence = sequence(epoch, token);
@@ -596,6 +635,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             backoff();
         }
         issued += __popcll(accepted);
+        PCIE_EP_PROFILE(profile.first(kProfileFirstTicketNs); profile.last(kProfileLastTicketNs);)
         // Every accepted entry is captured in a ticket: return the credits, one
         // store per source for the whole run (entries are consumed in order).  The
         // payload ACK and the ticket ring entry are separate resources.
@@ -609,6 +649,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             raise_abort(q);
             device_store(&q.rx_finished[channel].value, 1u);
         }
+        PCIE_EP_PROFILE(profile.save(state.profiling, state.z.dims.channels + channel, lane);)
         return;
     }
     // RX is finished when every ticket has been retired by a worker.
@@ -617,6 +658,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         if (broadcast_first(int(device_load(&q.rx_retired[channel].value))) >= issued && issued >= total) break;
         backoff();
     }
+    PCIE_EP_PROFILE(profile.first(kProfileWorkersDoneNs); profile.values[kProfileItems] = uint64_t(issued);)
     if (lane == 0) {
         atomicAdd(reinterpret_cast<unsigned long long*>(state.channel_stats + channel * kStatFields + kStatRxNotReady),
                   static_cast<unsigned long long>(not_ready));
@@ -627,6 +669,7 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
                   static_cast<unsigned long long>(ring_waits));
         device_store(&q.rx_finished[channel].value, 1u);
     }
+    PCIE_EP_PROFILE(profile.last(kProfileFinishedNs); profile.save(state.profiling, state.z.dims.channels + channel, lane);)
 }
 
 // ---------------------------------------------------------------------------------------
@@ -719,7 +762,7 @@ struct WorkerCounters {
 // into its host slot and publishes it.  Returns false when the wavefront must stop.
 template <bool kFp8, bool kVector>
 __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, const Deadline& deadline,
-                       WorkerCounters& counters) {
+                       WorkerCounters& counters PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
     const int endpoint_count = z.endpoints;
@@ -756,6 +799,7 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
         }
         if (targeted && my_descriptor >= descriptors) credit_ok = false;
         bool stop = false;
+        PCIE_EP_PROFILE(const uint64_t flow_begin = sampled ? profile.now() : 0;)
         while (true) {
             if (!slot_ok) slot_ok = host_load(ack_at(z, own, channel, slot, lane)) == previous_sequence;
             if (!credit_ok) credit_ok = credit_covers(host_load(credit_at(z, own, channel, lane)), epoch, my_descriptor, descriptors);
@@ -769,6 +813,7 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
         }
         if (stop) return false;
         compiler_barrier();
+        PCIE_EP_PROFILE(const uint64_t copy_begin = sampled ? profile.now() : 0; if (sampled) profile.add(kProfileTxFlowWaitSum, copy_begin - flow_begin);)
 
         // Slot metadata: composed in this wavefront's LDS scratch, then copied out
         // as consecutive dwords.  Weights are the live ones of this dispatch.
@@ -798,6 +843,7 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
         // Every lane's payload and metadata stores have been acknowledged before
         // any lane publishes a descriptor (the counters are wave-wide).
         wait_memory_ops();
+        PCIE_EP_PROFILE(if (sampled) profile.add(kProfileTxCopySum, profile.now() - copy_begin);)
         if (targeted) {
             // READY, slot and token in one 16-byte store: nothing to order inside the entry.
             const uint64_t ready = sequence(epoch, my_descriptor);
@@ -824,7 +870,7 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 // wavefront must stop.
 template <bool kFp8, bool kVector>
 __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters,
-                       bool& prefixes_known) {
+                       bool& prefixes_known PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
@@ -856,6 +902,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
             int(device_load(&q.rx_retired[channel].value)) < channel_ordinal)
             atomicAdd(reinterpret_cast<unsigned long long*>(state.receive_expand_overlap + channel * 2), 1ull);
 
+        PCIE_EP_PROFILE(const uint64_t request_begin = sampled ? profile.now() : 0;)
         // Metadata first (it arrives first), payload right behind it.
         const u32x4 meta_vector = host_load_b128(slot_meta, uint32_t(lane) * 16u);  // 16 bytes per lane; out of range reads as 0
 
@@ -893,6 +940,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 
         // The row has been requested; where it goes depends on the receive prefixes,
         // which may still be on their way in the first microseconds of the kernel.
+        PCIE_EP_PROFILE(const uint64_t prefix_begin = sampled ? profile.now() : 0;)
         while (!prefixes_known) {
             const int verdict = receive_prefix_verdict(state, epoch, lane);
             if (verdict < 0 || broadcast_first(aborted(q) ? 1 : 0)) return false;
@@ -900,6 +948,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
             else backoff();
         }
 
+        PCIE_EP_PROFILE(if (sampled) profile.add(kProfileRxPrefixWaitSum, profile.now() - prefix_begin);)
         // Destination rows, one lane per branch.  Everything the row numbers are
         // made of comes from the peer: the token must be addressed to this rank and
         // its ordinals must lie inside the counts that peer announced, or a store
@@ -964,6 +1013,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
                 if (last_pass) {
                     // All loads of the staged row have returned: release the host slot.
                     if (lane == 0) host_store_release(slot_ack, payload_sequence);
+                    PCIE_EP_PROFILE(if (sampled) { wait_memory_ops(); profile.add(kProfileRxRequestSum, profile.now() - request_begin); })
                 }
                 if constexpr (kFp8) {
                     // 16 codes -> 16 BF16 (two 16-byte vectors); expanded in place from the top.
@@ -1051,6 +1101,7 @@ __device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
             }
         }
         ++counters.reads;
+        PCIE_EP_PROFILE(if (sampled) profile.add(kProfileRxScatterSum, profile.now() - request_begin);)
         fence_lds();  // scratch is reused by the next ticket
         if (lane == 0) device_add(&q.rx_retired[channel].value, 1u);
     }
@@ -1097,6 +1148,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
     const uint64_t epoch = *state.epoch;
     Deadline deadline(now_ticks());
     WorkerCounters counters;
+    PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz); uint64_t idle_begin = 0; int rows_moved = 0;)
     bool prefixes_known = false;
     const int lead = int(kTxLeadBytes / int64_t(state.z.meta_offset + state.z.meta_bytes));
     uint64_t idle_since = 0;  // 0: the last look found work
@@ -1142,11 +1194,14 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
         choice = broadcast_first(choice);
         if (choice < 0) break;
         if (choice == 0) {
+            PCIE_EP_PROFILE(if (!idle_begin) idle_begin = profile.now();)
             backoff();
             continue;
         }
+        PCIE_EP_PROFILE(if (idle_begin) { profile.add(kProfileIdleSum, profile.now() - idle_begin); idle_begin = 0; })
         const bool transmit = choice == 1;
         QueueCounter& head = transmit ? q.tx_head : q.rx_head;
+        PCIE_EP_PROFILE(profile.first(kProfileFirstClaimNs); const uint64_t claim_begin = profile.now();)
         const int ticket_index = claim_ticket(head, lane);
         // Several wavefronts may have seen the same backlog: a claim beyond the last
         // ticket of the dispatch is simply dropped, an earlier one waits for its tag.
@@ -1154,8 +1209,11 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
             if (broadcast_first(aborted(q) ? 1 : 0)) break;
             continue;
         }
-        const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters)
-                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, prefixes_known);
+        PCIE_EP_PROFILE(profile.add(kProfileTicketWaitSum, profile.now() - claim_begin); const bool sampled = rows_moved++ % kProfileSampleStride == 0;
+                        if (sampled) profile.add(transmit ? kProfileSampledTxRows : kProfileSampledRxRows); profile.add(transmit ? kProfileTxRows : kProfileRxRows);)
+        const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters PCIE_EP_PROFILE(, profile, sampled))
+                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, prefixes_known PCIE_EP_PROFILE(, profile, sampled));
+        PCIE_EP_PROFILE(profile.last(kProfileLastRowNs);)
         if (!go_on) break;
     }
     // Workers serve every channel; their counts go to channel 0's row of the
@@ -1170,6 +1228,7 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
         }
         if (counters.reads) atomicAdd(stats + kStatHostReads, static_cast<unsigned long long>(counters.reads));
     }
+    PCIE_EP_PROFILE(profile.values[kProfileItems] = uint64_t(rows_moved); profile.save(state.profiling, 2 * state.z.dims.channels + order, lane);)
 }
 
 // Workgroup b < C is the control workgroup of channel b (wavefront 0 TX control,
@@ -1220,6 +1279,19 @@ int transport_threads(const DeviceState& state) {
     const int payload = state.tx_waves + state.rx_waves;
     const int control = state.worker_groups > 0 ? 2 : 2 + payload;
     return (control > payload ? control : payload) * kWave;
+}
+
+// How many transport workgroups one compute unit holds at once (registers, LDS and
+// wavefront slots of the instantiation that `state` selects).
+hipError_t transport_workgroups_per_unit(const DeviceState& state, int* per_unit) {
+    const int threads = transport_threads(state);
+    if (threads > kTransportMaxThreads) return hipErrorInvalidValue;
+    const bool fp8 = state.z.dims.wire_fp8 != 0;
+    const bool vector = fp8 ? state.z.dims.hidden % 16 == 0 : state.z.dims.hidden % 8 == 0;
+    if (fp8 && vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, true>, threads, 0);
+    if (fp8) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, false>, threads, 0);
+    if (vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, true>, threads, 0);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, false>, threads, 0);
 }
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {

@@ -10,7 +10,12 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
-LIBRARY_PATH = Path(__file__).resolve().parent / "lib" / "libpcie_ep_amd.so"
+import os
+
+# PCIE_EP_PROFILING=1 selects the library built with per-role timing records
+# (python pcie-ep_amd/build.py --profiling); everything else is identical.
+LIBRARY_PATH = Path(__file__).resolve().parent / "lib" / (
+    "libpcie_ep_amd_profiling.so" if os.environ.get("PCIE_EP_PROFILING") == "1" else "libpcie_ep_amd.so")
 
 E_INVALID, E_HIP, E_STATE, E_TIMEOUT, E_PROTOCOL = -1, -2, -3, -4, -5
 
@@ -80,6 +85,7 @@ _PROTOTYPES = {
     "pcie_ep_runtime_destroy": (C.c_int, [C.c_void_p]),
     "pcie_ep_dispatch": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
     "pcie_ep_dispatch_static_scratch": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
+    "pcie_ep_transport_residency": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "pcie_ep_expand_unique": (C.c_int, [C.c_void_p, C.POINTER(DispatchArgs), C.c_void_p]),
     "pcie_ep_set_test_delays": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64]),
     "pcie_ep_set_test_prefix_delay_ns": (C.c_int, [C.c_void_p, C.c_uint64]),
@@ -93,6 +99,8 @@ _PROTOTYPES = {
     "pcie_ep_host_signal_load": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64)]),
     "pcie_ep_quantize_fp8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "pcie_ep_dequantize_fp8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "pcie_ep_profile_shape": (C.c_int, [C.c_void_p] + [C.POINTER(C.c_int32)] * 4),
+    "pcie_ep_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_int64)]),
     "pcie_ep_set_kernel_timing": (C.c_int, [C.c_void_p, C.c_int32]),
     "pcie_ep_get_kernel_times": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "pcie_ep_measure_pinned_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),

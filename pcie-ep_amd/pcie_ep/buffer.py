@@ -165,7 +165,9 @@ class HostStagedEPBuffer:
         rings.  Default: every rank on the GPU's node, i.e. one domain.
         ``comm_stream_cus`` > 0 confines the dispatch kernels to that many compute
         units (``pcie_ep.streams``), so that compute kernels on a stream masked to
-        the remaining units run undisturbed while a dispatch is in flight; 64 units
+        the remaining units run undisturbed while a dispatch is in flight.  The units
+        must hold every control and payload workgroup of a dispatch at once (checked
+        here, ``ValueError`` otherwise: 80 workgroups at the defaults); 32 units
         carry the dispatch at full link rate.
         """
         if not torch.cuda.is_available():
@@ -215,6 +217,17 @@ class HostStagedEPBuffer:
                                      self.device, peer_threads=threads, staging_numa_node=staging_numa_node,
                                      tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups,
                                      rank_numa_nodes=rank_numa_nodes)
+        if comm_stream_cus:
+            # Control and payload workgroups wait for each other through device memory:
+            # the masked units must hold all of them at once, or every dispatch would
+            # end in the ring-progress timeout.
+            needed, resident = self.runtime.transport_residency(comm_stream_cus)
+            if resident < needed:
+                per_unit = max(1, resident // comm_stream_cus)
+                self.runtime.close()
+                self.runtime = None
+                raise ValueError(f"comm_stream_cus={comm_stream_cus} holds {resident} transport workgroups at once but a dispatch needs "
+                                 f"{needed} running together; use at least {-(-needed // per_unit)} compute units")
         self.peers = PeerGroup(self.runtime) if threads > 0 and num_ranks > 1 else None
 
     def _refuse_unsupported_world(self, group: Any, control_group: Any, reuse_comm: bool) -> None:

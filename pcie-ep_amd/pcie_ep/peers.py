@@ -14,7 +14,7 @@ import torch
 from . import _native
 
 (FAULT_NONE, FAULT_NO_COUNTS_READY, FAULT_NO_COUNTS_CONSUMED, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE, FAULT_RANK_ORDINAL,
- FAULT_EXPERT_ORDINAL) = range(7)
+ FAULT_EXPERT_ORDINAL, FAULT_SLOT_RANGE) = range(8)
 
 
 class PeerGroup:

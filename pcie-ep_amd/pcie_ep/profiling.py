@@ -1,0 +1,97 @@
+"""Per-role timing records of a dispatch (profiling builds of the library only).
+
+Counterpart of the reference's ``handle.profiling`` tensor and its schema
+(docs/pcie-ep/profiling-instrumentation.md:40-92): one record of 32 int64 per
+role wavefront, written once when the role ends.  Build the variant with
+``python pcie-ep_amd/build.py --profiling`` and select it with
+``PCIE_EP_PROFILING=1`` before importing ``pcie_ep``.
+
+Rows: TX control ``[0, C)``, RX control ``[C, 2C)``, payload wavefronts
+``[2C, 2C + W)``, prologue leader ``[2C + W]``.  Stamps (``*_ns``) are
+nanoseconds of the device wall clock, sums are accumulated nanoseconds; a zero
+stamp means the event did not happen.  Intervals of different roles overlap.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict
+
+import numpy as np
+
+from . import _native
+
+COMMON = ("enter_ns", "exit_ns", "total_ns", "items")
+CONTROL = COMMON + ("first_ticket_ns", "last_ticket_ns", "workers_done_ns", "drained_ns", "finished_ns", "polls", "poll_misses",
+                    "poll_sum", "health_scans", "health_sum", "counts_known_ns", "gate_open_ns", "prefix_enter_ns",
+                    "prefix_counts_ready_ns", "prefix_mailbox_ns", "prefix_published_ns")
+WORKER = COMMON + ("first_claim_ns", "last_row_ns", "tx_rows", "rx_rows", "sampled_tx_rows", "sampled_rx_rows", "ticket_wait_sum",
+                   "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum")
+PROLOGUE = COMMON + ("layout_ns", "totals_ns", "verdict_ns", "mailbox_free_ns", "mailbox_acked_ns", "counts_ready_ns")
+
+
+def read(runtime) -> Dict[str, np.ndarray]:
+    """Records of the runtime's last dispatch (waits for the device), split by role."""
+    lib = _native.library()
+    rows, fields, channels, wavefronts = (C.c_int32() for _ in range(4))
+    _native.check(lib.pcie_ep_profile_shape(runtime.handle, C.byref(rows), C.byref(fields), C.byref(channels), C.byref(wavefronts)),
+                  invalid=RuntimeError)
+    if rows.value == 0:
+        raise RuntimeError("the loaded library has no profiling records: build with --profiling and set PCIE_EP_PROFILING=1")
+    table = np.zeros((rows.value, fields.value), dtype=np.int64)
+    _native.check(lib.pcie_ep_profile_read(runtime.handle, table.ctypes.data_as(C.POINTER(C.c_int64))), invalid=RuntimeError)
+    c, w = channels.value, wavefronts.value
+    return {"tx_control": table[:c], "rx_control": table[c : 2 * c], "workers": table[2 * c : 2 * c + w], "prologue": table[2 * c + w]}
+
+
+def _col(rows: np.ndarray, names, name: str) -> np.ndarray:
+    return rows[..., names.index(name)]
+
+
+def timeline(records: Dict[str, np.ndarray]) -> Dict[str, float]:
+    """Key events of one dispatch in microseconds after the prologue's entry
+    (min over roles for 'first' events, max for 'last' ones)."""
+    pro, txc, rxc, wrk = records["prologue"], records["tx_control"], records["rx_control"], records["workers"]
+    zero = int(_col(pro, PROLOGUE, "enter_ns"))
+
+    def first(values) -> float:
+        values = np.asarray(values).reshape(-1)
+        values = values[values > 0]
+        return float("nan") if values.size == 0 else (int(values.min()) - zero) / 1e3
+
+    def last(values) -> float:
+        values = np.asarray(values).reshape(-1)
+        values = values[values > 0]
+        return float("nan") if values.size == 0 else (int(values.max()) - zero) / 1e3
+
+    def per(total, count) -> float:
+        count = int(np.sum(count))
+        return float("nan") if count == 0 else float(np.sum(total)) / count / 1e3
+
+    out = {f"prologue.{name[:-3]}": first(_col(pro, PROLOGUE, name)) for name in PROLOGUE[4:] + ("exit_ns",)}
+    active = wrk[_col(wrk, WORKER, "items") > 0]
+    out.update({
+        "transport.first_role_enter": first(np.concatenate([_col(txc, CONTROL, "enter_ns"), _col(rxc, CONTROL, "enter_ns"), _col(wrk, WORKER, "enter_ns")])),
+        "prefix.enter": first(_col(rxc, CONTROL, "prefix_enter_ns")), "prefix.counts_ready_seen": first(_col(rxc, CONTROL, "prefix_counts_ready_ns")),
+        "prefix.mailboxes_returned": first(_col(rxc, CONTROL, "prefix_mailbox_ns")), "prefix.published": first(_col(rxc, CONTROL, "prefix_published_ns")),
+        "rx.first_gate_open": first(_col(rxc, CONTROL, "gate_open_ns")), "rx.first_ticket": first(_col(rxc, CONTROL, "first_ticket_ns")),
+        "rx.last_ticket": last(_col(rxc, CONTROL, "last_ticket_ns")), "rx.counts_known_first": first(_col(rxc, CONTROL, "counts_known_ns")),
+        "rx.rows_scattered_last": last(_col(rxc, CONTROL, "workers_done_ns")), "rx.finished_last": last(_col(rxc, CONTROL, "finished_ns")),
+        "rx.descriptor_poll_us": per(_col(rxc, CONTROL, "poll_sum"), _col(rxc, CONTROL, "polls")),
+        "rx.polls": float(np.sum(_col(rxc, CONTROL, "polls"))), "rx.poll_misses": float(np.sum(_col(rxc, CONTROL, "poll_misses"))),
+        "tx.first_ticket": first(_col(txc, CONTROL, "first_ticket_ns")), "tx.last_ticket": last(_col(txc, CONTROL, "last_ticket_ns")),
+        "tx.rows_published_last": last(_col(txc, CONTROL, "workers_done_ns")), "tx.drained_last": last(_col(txc, CONTROL, "drained_ns")),
+        "tx.finished_last": last(_col(txc, CONTROL, "finished_ns")), "tx.drain_poll_us": per(_col(txc, CONTROL, "poll_sum"), _col(txc, CONTROL, "polls")),
+        "tx.drain_polls": float(np.sum(_col(txc, CONTROL, "polls"))), "tx.drain_misses": float(np.sum(_col(txc, CONTROL, "poll_misses"))),
+        "workers.first_claim": first(_col(wrk, WORKER, "first_claim_ns")), "workers.last_row_end": last(_col(wrk, WORKER, "last_row_ns")),
+        "workers.active": float(active.shape[0]),
+        "workers.ticket_wait_us": per(_col(wrk, WORKER, "ticket_wait_sum"), _col(wrk, WORKER, "items")),
+        "workers.rx_request_to_data_us": per(_col(wrk, WORKER, "rx_request_sum"), _col(wrk, WORKER, "sampled_rx_rows")),
+        "workers.rx_request_to_stores_us": per(_col(wrk, WORKER, "rx_scatter_sum"), _col(wrk, WORKER, "sampled_rx_rows")),
+        "workers.rx_prefix_wait_us": per(_col(wrk, WORKER, "rx_prefix_wait_sum"), _col(wrk, WORKER, "sampled_rx_rows")),
+        "workers.tx_flow_wait_us": per(_col(wrk, WORKER, "tx_flow_wait_sum"), _col(wrk, WORKER, "sampled_tx_rows")),
+        "workers.tx_copy_to_ack_us": per(_col(wrk, WORKER, "tx_copy_sum"), _col(wrk, WORKER, "sampled_tx_rows")),
+        "workers.idle_us_mean": per(_col(wrk, WORKER, "idle_sum"), np.array([max(1, wrk.shape[0])])),
+        "transport.last_role_exit": last(np.concatenate([_col(txc, CONTROL, "exit_ns"), _col(rxc, CONTROL, "exit_ns"), _col(wrk, WORKER, "exit_ns")])),
+    })
+    return out

@@ -314,6 +314,14 @@ class NativeRuntime:
         stream = torch.cuda.current_stream(self.device).cuda_stream
         _native.check(self._lib.pcie_ep_expand_unique(self._require(), C.byref(arguments), C.c_void_p(stream)), invalid=RuntimeError)
 
+    def transport_residency(self, compute_units: int = 0) -> tuple:
+        """(workgroups of one dispatch that must run at once, workgroups that
+        ``compute_units`` units - 0 = the device - hold at once)."""
+        needed, resident = C.c_int32(), C.c_int32()
+        _native.check(self._lib.pcie_ep_transport_residency(self._require(), compute_units, C.byref(needed), C.byref(resident)),
+                      invalid=RuntimeError)
+        return int(needed.value), int(resident.value)
+
     def set_kernel_timing(self, enable: bool) -> None:
         _native.check(self._lib.pcie_ep_set_kernel_timing(self._require(), int(enable)), invalid=RuntimeError)
 

@@ -16,7 +16,7 @@ import torch
 
 from helpers import make_inputs, run_dispatch, verify_dispatch
 from pcie_ep.peers import (FAULT_EXPERT_ORDINAL, FAULT_NO_COUNTS_CONSUMED, FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_RANK_ORDINAL,
-                           FAULT_WRONG_SEQUENCE)
+                           FAULT_SLOT_RANGE, FAULT_WRONG_SEQUENCE)
 from test_gpu_dispatch import make_buffer
 
 pytestmark = pytest.mark.gpu
@@ -93,6 +93,17 @@ def test_out_of_range_ordinals_from_a_peer_are_code_18(inputs, fault, expand):
     with small_buffer() as buffer:
         buffer.peers.inject_fault(4, fault)
         print(f"case: rank 4 sends an ordinal beyond its announced counts (fault {fault}, expand={expand})", flush=True)
+        failing_dispatch(buffer, inputs, 18, expand=expand)
+
+
+@pytest.mark.parametrize("expand", [True, False])
+def test_out_of_range_slot_in_a_descriptor_is_code_18(inputs, expand):
+    """A descriptor that names a payload slot beyond the ring would make the GPU
+    read outside the pinned segment: RX control refuses it before any ticket is
+    written, so no row is read and nothing is ACKed."""
+    with small_buffer() as buffer:
+        buffer.peers.inject_fault(2, FAULT_SLOT_RANGE)
+        print(f"case: rank 2 publishes a descriptor with slot == payload_slots (expand={expand})", flush=True)
         failing_dispatch(buffer, inputs, 18, expand=expand)
 
 
