@@ -43,6 +43,7 @@ HBM_PEAK_GBPS = 8000.0
 COPY_BYTES = 1 << 30  # calibration copy: 1 GiB read + 1 GiB written
 HOST_COPY_BYTES = 1 << 29  # kernel-driven pinned copy: 512 MiB each way
 BIT_EXACT = "bit-exact vs oracle"
+SPLIT_LAUNCH = False  # --split-launch: the prologue as a kernel of its own in front of the transport kernel
 
 
 def log(*items) -> None:
@@ -62,7 +63,7 @@ def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000, graph=Fals
                               fuse_receive_expand=fuse, receive_expand_mode="pipelined" if fuse else "scalar", timeout_ms=timeout_ms,
                               enable_graph=graph)
     return HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
-                              num_ranks=WORLD, rank=0)
+                              num_ranks=WORLD, rank=0, split_launch=SPLIT_LAUNCH)
 
 
 def set_peers(buffer, inputs):
@@ -394,10 +395,15 @@ def main() -> int:
                              "graph-replay / restaged sub-records); what the profiler runs use")
     parser.add_argument("--expand-only", action="store_true",
                         help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
+    parser.add_argument("--split-launch", action="store_true",
+                        help="run the prologue as a kernel of its own in front of the transport kernel (default: one launch per dispatch "
+                             "wherever the prologue fits into the transport launch)")
     parser.add_argument("--role-timeline", type=str, default="",
                         help="comma-separated token counts: print the per-role timeline of the dispatch at those sizes and exit "
                              "(needs the profiling build: python pcie-ep_amd/build.py --profiling)")
     args = parser.parse_args()
+    global SPLIT_LAUNCH
+    SPLIT_LAUNCH = args.split_launch
     if args.role_timeline:
         os.environ["PCIE_EP_PROFILING"] = "1"
     if args.gpus != 1:

@@ -64,7 +64,9 @@ typedef struct pcie_ep_config {
     int32_t replica_slots;      /* R per (channel, NUMA domain), relay mode */
     int32_t relay_workers_per_numa; /* host relay threads per NUMA domain, 1..channels */
     int32_t relay_cpu_count;    /* entries of relay_cpus in use; 0 = any CPU the process may run on */
-    int32_t reserved[5];
+    int32_t split_launch;       /* 0: one launch per dispatch where the prologue fits into the transport launch (top-k <= 8, default
+                                   launch shape, at most 64 chunks of 256 tokens); 1: always a prologue launch of its own */
+    int32_t reserved[4];
     int32_t rank_numa_nodes[16];/* physical NUMA node of every rank, -1 = unknown (one domain) */
     int32_t relay_cpus[64];     /* CPUs the relay workers may be pinned to */
     uint64_t relay_delay_ns;    /* test hook: delay before each relay copy */

@@ -76,6 +76,11 @@ struct alignas(256) TransportQueues {
     QueueCounter abort;             // value != 0: every role exits
     QueueCounter local_head;        // own tokens (then padding gaps) claimed for the local bypass
     QueueCounter finished;          // role wavefronts that have ended; the last one reduces the statistics
+    // Prologue inside the transport launch: value = epoch_flag(epoch) once the epoch begin has cleared the
+    // diagnostics and reset the queues (begun) / has found no abort word set and the previous count mailbox
+    // consumed (verdict) / the leader has published the counts and the whole plan is in memory (plan_ready);
+    // plan_chunks counts the chunks other than the leader's whose part of the plan is in memory.
+    QueueCounter begun, verdict, plan_ready, plan_chunks;
     QueueCounter rx_retired[kMaxChannels], tx_retired[kMaxChannels], rx_finished[kMaxChannels];
     uint64_t rx_ready[kRing], rx_taken[kRing];  // sequence(epoch, n): entry n % kRing holds / has been copied out
     uint64_t tx_ready[kRing], tx_taken[kRing];
@@ -99,6 +104,8 @@ struct DeviceState {
     int reuse_plan;
     int counts_ack_skip_source;
     int overlap_diagnostic;  // fill receive_expand_overlap (count, completion watermark); 0 leaves it zero
+    int fused;               // 1: the prologue runs as the first workgroups of the transport launch
+    int prologue_chunks;     // token chunks of this dispatch's layout (0 when a cached plan is reused)
     uint64_t timeout_ticks;
     uint64_t clock_khz;  // rate of wall_clock64() on this device (hipDeviceAttributeWallClockRate)
     uint64_t* epoch;
@@ -174,6 +181,16 @@ __device__ __forceinline__ int64_t ticks_to_ns(const DeviceState& state, uint64_
     return int64_t(ticks / khz * 1000000ull + ticks % khz * 1000000ull / khz);
 }
 __device__ __forceinline__ void backoff() { __builtin_amdgcn_s_sleep(8); }
+// Epoch of the running dispatch.  With the prologue in a launch of its own the epoch word has been advanced when
+// the transport kernel starts; inside one launch it still holds the previous epoch until the last role ends.
+__device__ __forceinline__ uint64_t dispatch_epoch(const DeviceState& state) { return *state.epoch + uint64_t(state.fused); }
+// Workgroups in front of the transport roles when the prologue rides in the transport launch: the epoch begin and one
+// per chunk of tokens (one, the leader, also when there is nothing to lay out).
+__host__ __device__ __forceinline__ int fused_prologue_groups(const DeviceState& state) {
+    return state.fused ? 1 + (state.prologue_chunks > 1 ? state.prologue_chunks : 1) : 0;
+}
+// 32-bit value an epoch-tagged flag word carries (epochs stay below 2^32; the one beyond, which only ends in error 20, still gets a value of its own).
+__device__ __forceinline__ uint32_t epoch_flag(uint64_t epoch) { return uint32_t(epoch) + uint32_t(epoch >> 32) * 0x9E3779B9u; }
 
 #if PCIE_EP_ENABLE_PROFILING
 // Fields of one role's record.  Times are nanoseconds of the device's wall clock
@@ -219,9 +236,17 @@ enum PrologueProfileField : int {
     kPrologueMailboxFreeNs,    // previous count mailbox seen consumed by every peer
     kPrologueMailboxAckedNs,   // count mailbox stores acknowledged by the host
     kPrologueCountsReadyNs,    // counts_ready stored
+    kPrologueBegunNs,          // diagnostics cleared, queues reset (and, inside the transport launch, announced)
+    kPrologueRoutesNs,         // route ids loaded and checked, hit masks requested
+    kPrologueMasksNs,          // hit masks and channel counts of the chunk complete
+    kPrologueChunkTotalsNs,    // chunk totals stored (single chunk: the plan's totals)
+    kProloguePlanReadyNs,      // inside the transport launch: plan_ready announced
 };
-// Rows of the table: TX controls [0, C), RX controls [C, 2C), payload wavefronts, prologue leader.
-__host__ __device__ inline int profile_rows(int channels, int payload_wavefronts) { return 2 * channels + payload_wavefronts + 1; }
+// Rows of the table: TX controls [0, C), RX controls [C, 2C), payload wavefronts, prologue leader, epoch begin
+// (a record of its own only where the prologue rides in the transport launch; otherwise the leader's holds its stamps),
+// producer of the receive prefixes (a record of its own only where it is a wavefront of its own; otherwise the
+// prefix fields of the elected RX control's record hold its stamps).
+__host__ __device__ inline int profile_rows(int channels, int payload_wavefronts) { return 2 * channels + payload_wavefronts + 3; }
 struct RoleProfile {
     uint64_t values[kProfileFields] = {};
     uint64_t khz;
@@ -243,7 +268,7 @@ struct RoleProfile {
 };
 #endif
 
-__device__ inline void test_delay(uint64_t ticks) {
+__device__ __forceinline__ void test_delay(uint64_t ticks) {
     if (!ticks) return;
     const uint64_t start = now_ticks();
     while (now_ticks() - start < ticks) __builtin_amdgcn_s_sleep(16);
@@ -389,6 +414,13 @@ __device__ __forceinline__ uint32_t device_load_b32(__amdgpu_buffer_rsrc_t resou
 __device__ __forceinline__ void device_store_b32(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, uint32_t value) {
     __builtin_amdgcn_raw_buffer_store_b32(value, resource, int(byte_offset), 0, kDevicePolicy);
 }
+// Sixteen bytes as one write-through transaction where four 4-byte ones would each travel to memory alone.
+__device__ __forceinline__ void device_store_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, u32x4 value) {
+    __builtin_amdgcn_raw_buffer_store_b128(value, resource, int(byte_offset), 0, kDevicePolicy);
+}
+__device__ __forceinline__ void plain_store_b128(__amdgpu_buffer_rsrc_t resource, uint32_t byte_offset, u32x4 value) {
+    __builtin_amdgcn_raw_buffer_store_b128(value, resource, int(byte_offset), 0, 0);
+}
 
 // Streaming row accesses in device memory: buffer instructions with the non-temporal
 // policy.  Lanes beyond the resource's size read zero / are dropped, so rows need no
@@ -417,11 +449,11 @@ __device__ __forceinline__ int64_t load_error_code(const DeviceState& state) {
 
 // First error wins; context fields follow the reference
 // (advanced_common.cuh:289-295: errors[1] = local rank, errors[2] = epoch).
-__device__ inline void record_error(const DeviceState& state, int code, int64_t context = -1, int64_t detail = -1) {
+__device__ __forceinline__ void record_error(const DeviceState& state, int code, int64_t context = -1, int64_t detail = -1) {
     unsigned long long expected = 0;
     if (atomicCAS(reinterpret_cast<unsigned long long*>(state.errors), expected, static_cast<unsigned long long>(code)) == 0ull) {
         state.errors[1] = context >= 0 ? context : state.local_rank;
-        state.errors[2] = detail >= 0 ? detail : int64_t(*state.epoch);
+        state.errors[2] = detail >= 0 ? detail : int64_t(dispatch_epoch(state));
     }
 }
 
@@ -442,7 +474,7 @@ __device__ __forceinline__ const uint64_t* abort_flag_at(const SegmentLayout& z,
     if (flag <= z.dims.channels) return signal_at(segment, z.channel_abort_offset, flag - 1);
     return signal_at(segment, z.relay_failed_offset, flag - 1 - z.dims.channels);
 }
-__device__ inline bool any_abort_wave(const DeviceState& state, int lane, int slice = 0, int slices = 1) {
+__device__ __forceinline__ bool any_abort_wave(const DeviceState& state, int lane, int slice = 0, int slices = 1) {
     const int per_rank = abort_flags_per_rank(state.z);
     const int flags = state.z.dims.num_ranks * per_rank;
     bool aborted = false;
@@ -476,7 +508,7 @@ struct HealthCheck {
     uint64_t interval;
     uint64_t limit;
     int member, members, scans;
-    __device__ HealthCheck(const DeviceState& state, uint64_t begin, bool progress_wait = false, int member_ = 0, int members_ = 1)
+    __device__ __forceinline__ HealthCheck(const DeviceState& state, uint64_t begin, bool progress_wait = false, int member_ = 0, int members_ = 1)
         : start(begin), member(member_), members(members_), scans(0) {
         const uint64_t cap = state.clock_khz;  // one millisecond
         const uint64_t eighth = state.timeout_ticks / 8;
@@ -484,7 +516,7 @@ struct HealthCheck {
         next_scan = begin + interval;
         limit = progress_wait ? progress_timeout_ticks(state) : state.timeout_ticks;
     }
-    __device__ bool poll(const DeviceState& state, int lane) {
+    __device__ __forceinline__ bool poll(const DeviceState& state, int lane) {
         const uint64_t now = now_ticks();
         if (now - start > limit) return true;
         // `now` differs slightly per lane; take lane 0's verdict for the scan.

@@ -51,6 +51,13 @@ static_assert((2 + kMaxTxWaves + kMaxRxWaves) * kWave <= kTransportMaxThreads, "
 hipError_t launch_prologue(const DeviceState& state, hipStream_t stream);
 size_t prologue_flag_bytes(const SegmentLayout& z);
 size_t prologue_scratch_bytes(const SegmentLayout& z);
+size_t prologue_lds_bytes(const SegmentLayout& z, int chunk_waves);
+int prologue_chunk_waves(const SegmentLayout& z);
+// Chunks of `tokens` tokens at `chunk_waves` wavefronts per chunk (0: the prologue kernel's own shape).
+int prologue_chunks(const SegmentLayout& z, int tokens, int chunk_waves);
+// Whether the prologue can run inside the transport launch (workgroups of `block_threads` threads);
+// launch_transport runs it there when DeviceState::fused is set, and launch_prologue is then not called.
+bool fused_prologue_fits(const SegmentLayout& z, int block_threads, int max_tokens);
 // Channel transport: control / TX / RX-scatter wavefront roles, the local bypass,
 // alignment-gap zeroing and the statistics reduction.
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream);

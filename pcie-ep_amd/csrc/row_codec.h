@@ -15,7 +15,7 @@ __device__ __forceinline__ float wave_max(float value) {
 
 // BF16 row copy.  kVector requires hidden % 8 == 0 and 16-byte aligned rows.
 template <bool kVector, bool kStreamOut>
-__device__ inline void copy_row(const uint16_t* input, uint16_t* output, int hidden, int lane) {
+__device__ __forceinline__ void copy_row(const uint16_t* input, uint16_t* output, int hidden, int lane) {
     if constexpr (kVector) {
         const int vectors = hidden / 8;
         const u32x4* source = reinterpret_cast<const u32x4*>(input);
@@ -45,7 +45,7 @@ struct HostCodes {
 
 // BF16 row from device memory into a host slot.
 template <bool kVector>
-__device__ inline void copy_row_to_host(const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int hidden, int lane) {
+__device__ __forceinline__ void copy_row_to_host(const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int hidden, int lane) {
     if constexpr (kVector) {
         const int vectors = hidden / 8;
         const u32x4* source = reinterpret_cast<const u32x4*>(input);
@@ -65,7 +65,7 @@ __device__ inline void copy_row_to_host(const uint16_t* input, __amdgpu_buffer_r
 
 // Returns the row scale.  kVector requires hidden % 16 == 0.
 template <bool kVector, typename Sink>
-__device__ inline float quantize_row(const uint16_t* input, const Sink& sink, int hidden, int lane) {
+__device__ __forceinline__ float quantize_row(const uint16_t* input, const Sink& sink, int hidden, int lane) {
     // Sweep 1: row amax in FP32.  Sweep 2 re-reads the row (it is L2 resident).
     float amax = 0.0f;
     if constexpr (kVector) {
@@ -129,7 +129,7 @@ __device__ __forceinline__ void dequantize_vector(const u32x4& codes, float scal
 }
 
 template <bool kVector>
-__device__ inline void dequantize_row(const uint8_t* codes, float scale, uint16_t* output, int hidden, int lane) {
+__device__ __forceinline__ void dequantize_row(const uint8_t* codes, float scale, uint16_t* output, int hidden, int lane) {
     if constexpr (kVector) {
         const int groups = hidden / 16;
         const u32x4* source = reinterpret_cast<const u32x4*>(codes);
@@ -148,7 +148,7 @@ __device__ inline void dequantize_row(const uint8_t* codes, float scale, uint16_
 // Store one BF16 row (already read into registers pass by pass) to every
 // destination row named by the lanes whose `my_row >= 0`.
 template <bool kVector>
-__device__ inline void scatter_row(const uint16_t* input, uint16_t* output_base, int hidden, int64_t my_row, int lane) {
+__device__ __forceinline__ void scatter_row(const uint16_t* input, uint16_t* output_base, int hidden, int64_t my_row, int lane) {
     const uint64_t destinations = __ballot(my_row >= 0);
     if (!destinations) return;
     if constexpr (kVector) {
@@ -189,7 +189,7 @@ __device__ inline void scatter_row(const uint16_t* input, uint16_t* output_base,
 }
 
 template <bool kVector>
-__device__ inline void zero_row(uint16_t* output, int hidden, int lane) {
+__device__ __forceinline__ void zero_row(uint16_t* output, int hidden, int lane) {
     if constexpr (kVector) {
         u32x4* destination = reinterpret_cast<u32x4*>(output);
         const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -204,7 +204,7 @@ __device__ inline void zero_row(uint16_t* output, int hidden, int lane) {
 // The prefixes are read with device-scope loads: inside the transport kernel
 // they were written by another wavefront of the same launch.
 template <bool kVector>
-__device__ inline void zero_padding_of_expert(const DeviceState& state, int expert, int lane) {
+__device__ __forceinline__ void zero_padding_of_expert(const DeviceState& state, int expert, int lane) {
     const int hidden = state.z.dims.hidden;
     const int64_t next = device_load(state.expert_offsets + expert + 1);
     const int64_t end = next < state.expanded_capacity ? next : state.expanded_capacity;
@@ -222,7 +222,7 @@ __device__ inline void zero_padding_of_expert(const DeviceState& state, int expe
 // original BF16 even on an FP8 wire (advanced_layout.cuh:217-248).  Returns
 // false when a destination row lies beyond the expanded capacity.
 template <bool kVector>
-__device__ inline bool local_token_rows(const DeviceState& state, int token, int lane) {
+__device__ __forceinline__ bool local_token_rows(const DeviceState& state, int token, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;

@@ -252,6 +252,7 @@ struct pcie_ep_runtime {
     std::unique_ptr<PeerEmulator> peers;
     uint64_t clock_khz = 100000;  // wall clock of the device, queried at creation
     unsigned char* static_scratch = nullptr;  // device address of `scratch` on this runtime's GPU
+    bool fused = false;  // the prologue rides in the transport launch (one kernel per dispatch)
     bool closed = false;
     uint64_t ticks_of_ns(uint64_t ns) const { return ns / 1000000 * clock_khz + ns % 1000000 * clock_khz / 1000000; }
     // Optional per-kernel timing with HIP events on the launch stream.
@@ -333,6 +334,8 @@ int build_state(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* a, DeviceState
     s.reuse_plan = a->reuse_plan ? 1 : 0;
     s.counts_ack_skip_source = rt->counts_ack_skip_source;
     s.overlap_diagnostic = s.fuse_expand && s.expand && rt->config.receive_expand_mode == 0;
+    s.fused = rt->fused ? 1 : 0;
+    s.prologue_chunks = (rt->fused && !a->reuse_plan) ? prologue_chunks(rt->z, a->num_tokens, transport_threads(s) / kWave) : 0;
     s.timeout_ticks = uint64_t(rt->config.timeout_ms) * rt->clock_khz;
     s.clock_khz = rt->clock_khz;
     s.epoch = rt->epoch;
@@ -449,6 +452,17 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     rt->tx_waves = shape.tx_waves;
     rt->rx_waves = shape.rx_waves;
     rt->worker_groups = shape.worker_groups;
+    {
+        DeviceState probe{};
+        probe.tx_waves = rt->tx_waves;
+        probe.rx_waves = rt->rx_waves;
+        probe.worker_groups = rt->worker_groups;
+        // One launch per dispatch wherever the prologue fits into the transport launch and the whole grid
+        // (epoch begin, prologue chunks of a full batch, control, payload and local-bypass workgroups) is resident at once.
+        const int block_threads = transport_threads(probe);
+        rt->fused = !config->split_launch && fused_prologue_fits(rt->z, block_threads, dims.max_tokens) &&
+                    1 + prologue_chunks(rt->z, dims.max_tokens, block_threads / kWave) + dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0) + 32 <= 256;
+    }
 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers
     // /dev/shm mappings: advanced_shared_memory.hpp:264-288).  First touch is
@@ -571,7 +585,7 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     const bool timed = rt->timing;
     rt->timing_valid = false;
     if (timed) HIP_TRY(hipEventRecord(rt->marks[0], stream));
-    HIP_TRY(launch_prologue(state, stream));
+    if (!state.fused) HIP_TRY(launch_prologue(state, stream));
     if (timed) HIP_TRY(hipEventRecord(rt->marks[1], stream));
     HIP_TRY(launch_transport(state, stream));
     if (timed) HIP_TRY(hipEventRecord(rt->marks[2], stream));
@@ -626,7 +640,7 @@ int pcie_ep_dispatch_static_scratch(pcie_ep_runtime* rt, const pcie_ep_dispatch_
     // tags, queue counters, prologue chunk flags) start from zero.  A fill kernel,
     // not a memset, so the call may be captured into a graph.
     HIP_TRY(launch_zero(base, carve.clear_bytes, stream));
-    HIP_TRY(launch_prologue(state, stream));
+    if (!state.fused) HIP_TRY(launch_prologue(state, stream));
     HIP_TRY(launch_transport(state, stream));
     if (state.expand && !state.fuse_expand) HIP_TRY(launch_expand(state, stream));
     if (!capturing) {
@@ -647,11 +661,13 @@ int pcie_ep_transport_residency(pcie_ep_runtime* rt, int32_t compute_units, int3
     probe.tx_waves = rt->tx_waves;
     probe.rx_waves = rt->rx_waves;
     probe.worker_groups = rt->worker_groups;
+    probe.fused = rt->fused ? 1 : 0;
     int per_unit = 0;
     HIP_TRY(transport_workgroups_per_unit(probe, &per_unit));
     // The control and payload workgroups wait for each other through device memory
     // and must run together; the local-bypass workgroups behind them may start late.
-    *needed = rt->z.dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0);
+    *needed = rt->z.dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0) +
+              (rt->fused ? 1 + std::max(1, prologue_chunks(rt->z, rt->z.dims.max_tokens, rt->tx_waves + rt->rx_waves)) : 0);
     *resident = per_unit * units;
     return 0;
 }

@@ -51,6 +51,7 @@
 //    per-channel statistics (:267-283).  The dispatch needs no kernel after this one.
 #include "device_common.h"
 #include "launch.h"
+#include "prologue_body.h"
 #include "row_codec.h"
 
 namespace pcie_ep {
@@ -70,11 +71,50 @@ struct WaveScratch {
 struct Deadline {
     uint64_t start;
     __device__ explicit Deadline(uint64_t begin) : start(begin) {}
-    __device__ bool expired(const DeviceState& state) const { return now_ticks() - start > progress_timeout_ticks(state); }
+    __device__ __forceinline__ bool expired(const DeviceState& state) const { return now_ticks() - start > progress_timeout_ticks(state); }
 };
 
 __device__ __forceinline__ bool aborted(TransportQueues& q) { return device_load(&q.abort.value) != 0; }
 __device__ __forceinline__ void raise_abort(TransportQueues& q) { device_store(&q.abort.value, 1u); }
+
+// Prologue inside this launch: a role may touch the queues and the diagnostics once
+// the epoch begin has cleared them.  One thread per workgroup polls (hundreds of
+// wavefronts polling one word would slow down the very stores they wait for).
+// Bounded: an epoch begin that never runs ends the role.
+__device__ __forceinline__ bool wait_for_begin(const DeviceState& state, TransportQueues& q) {
+    const uint32_t tag = epoch_flag(dispatch_epoch(state));
+    const uint64_t start = now_ticks();
+    // The word cannot be there in the first microsecond: stay off the memory the clearing goes to.
+    __builtin_amdgcn_s_sleep(48);
+    while (device_load(&q.begun.value) != tag) {
+        if (now_ticks() - start > state.timeout_ticks) return false;
+        __builtin_amdgcn_s_sleep(16);
+    }
+    return true;
+}
+// ... and read the route plan once the leader has published the counts and every
+// chunk's part of the plan is in memory.  False when the prologue failed (abort) or
+// never finished (timeout, recorded as a ring-progress error).
+__device__ __forceinline__ bool wait_for_plan(const DeviceState& state, TransportQueues& q, int lane) {
+    if (!state.fused) return true;
+    const uint32_t tag = epoch_flag(dispatch_epoch(state));
+    const uint64_t start = now_ticks();
+    while (true) {
+        int verdict = 0;
+        if (lane == 0) {
+            if (device_load(&q.plan_ready.value) == tag) verdict = 1;
+            else if (aborted(q)) verdict = -1;
+            else if (now_ticks() - start > progress_timeout_ticks(state)) {
+                record_error(state, kErrRingProgressWait);
+                raise_abort(q);
+                verdict = -1;
+            }
+        }
+        verdict = broadcast_first(verdict);
+        if (verdict) return verdict > 0;
+        backoff();
+    }
+}
 
 // Producer side: reserve `count` consecutive tickets (one fetch-add per wavefront).
 __device__ __forceinline__ int reserve_tickets(QueueCounter& tail, int count, int lane) {
@@ -94,7 +134,7 @@ __device__ __forceinline__ int claim_ticket(QueueCounter& head, int lane) {
     if (lane == 0) ticket = device_add(&head.value, 1u);
     return broadcast_first(int(ticket));
 }
-__device__ inline int wait_ticket(const DeviceState& state, TransportQueues& q, const uint64_t* ready, QueueCounter& head, int ticket,
+__device__ __forceinline__ int wait_ticket(const DeviceState& state, TransportQueues& q, const uint64_t* ready, QueueCounter& head, int ticket,
                                   uint64_t epoch, int lane, const Deadline& deadline) {
     while (true) {
         int action = 0;
@@ -122,11 +162,11 @@ __device__ inline int wait_ticket(const DeviceState& state, TransportQueues& q, 
 // elected by a device-scope CAS; it waits for every source's counts_ready,
 // folds the mailboxes in rank order and publishes a generation-valued READY.
 // ---------------------------------------------------------------------------------------
-__device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
+__device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, local = z.local_experts, channels = z.dims.channels;
     const int me = state.local_rank;
-    const uint64_t epoch = *state.epoch;
+    const uint64_t epoch = dispatch_epoch(state);
     const uint64_t start = now_ticks();
     HealthCheck health(state, start);
     PCIE_EP_PROFILE(profile.first(kProfilePrefixEnterNs);)
@@ -149,10 +189,14 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE
     // r's segment and hands it out by lane shuffle) - before the wait for the
     // sources, where it costs nothing - and the loads follow in one run.
     const char* const lane_segment = state.seg[lane < ranks ? lane : 0];
+    // Prologue in the same launch: the own counts are taken from the route plan in
+    // device memory once the leader has announced it, not from the own mailbox in
+    // host memory; the other sources' words are requested before that wait.
+    const bool own_from_plan = state.fused != 0;
     // The first look at every source's counts_ready is requested now; its value is
     // used after the address arithmetic below, which so runs inside its round trip.
     uint64_t first_look = 0;
-    if (lane < ranks) first_look = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
+    if (lane < ranks && !(own_from_plan && lane == me)) first_look = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
     const auto segment_of = [&](int rank) {
         const uint64_t bits = reinterpret_cast<uint64_t>(lane_segment);
         return reinterpret_cast<char*>(uint64_t(uint32_t(__shfl(int(uint32_t(bits)), rank))) | uint64_t(uint32_t(__shfl(int(uint32_t(bits >> 32)), rank))) << 32);
@@ -165,16 +209,19 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE
         const bool valid = index < channels * ranks;
         char* segment = segment_of(valid ? index % ranks : 0);
         expected_address[i] = valid ? mailbox_at(z, segment, me) + 1 + local + index / ranks : nullptr;
+        if (own_from_plan && valid && index % ranks == me) expected_address[i] = state.plan_chan_counts + (index / ranks) * ranks + me;
     }
     const int32_t* first_address[kMaxRanks];
 #pragma unroll
     for (int source = 0; source < kMaxRanks; ++source) {
         char* segment = segment_of(source < ranks ? source : 0);
         first_address[source] = (source < ranks && lane < local) ? mailbox_at(z, segment, me) + 1 + lane : nullptr;
+        if (own_from_plan && source == me && lane < local) first_address[source] = state.plan_counts + ranks + me * local + lane;
     }
     const int32_t* unique_address = lane < ranks ? mailbox_at(z, const_cast<char*>(lane_segment), me) : nullptr;
+    if (own_from_plan && lane == me) unique_address = state.plan_counts + me;
     // All sources are polled in parallel, one lane each.
-    bool ready = lane >= ranks || first_look == epoch;
+    bool ready = lane >= ranks || (own_from_plan && lane == me) || first_look == epoch;
     while (true) {
         if (__all(ready)) break;
         if (!ready) ready = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset)) == epoch;
@@ -183,24 +230,40 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE
             if (lane == 0) record_error(state, kErrCountsReadyWait);
             return false;
         }
+        // Nothing will come of this dispatch when the prologue of the same launch has failed.
+        if (state.fused && broadcast_first(aborted(*state.queues) ? 1 : 0)) return false;
         backoff();
     }
     wait_memory_ops();
     compiler_barrier();
     PCIE_EP_PROFILE(profile.first(kProfilePrefixCountsReadyNs);)
+    // Host words first (every word of the other sources, in one run) ...
     int unique = 0;
-    if (unique_address) unique = host_field_load_global(unique_address);
+    if (unique_address && !(own_from_plan && lane == me)) unique = host_field_load_global(unique_address);
     int expected_values[kExpectedPerLane];
 #pragma unroll
-    for (int i = 0; i < kExpectedPerLane; ++i) expected_values[i] = expected_address[i] ? host_field_load_global(expected_address[i]) : 0;
+    for (int i = 0; i < kExpectedPerLane; ++i)
+        expected_values[i] = (expected_address[i] && !(own_from_plan && (lane + i * kWave) % ranks == me)) ? host_field_load_global(expected_address[i]) : 0;
     int first_counts[kMaxRanks];
 #pragma unroll
-    for (int source = 0; source < kMaxRanks; ++source) first_counts[source] = first_address[source] ? host_field_load_global(first_address[source]) : 0;
+    for (int source = 0; source < kMaxRanks; ++source)
+        first_counts[source] = (first_address[source] && !(own_from_plan && source == me)) ? host_field_load_global(first_address[source]) : 0;
     // The reads are on the link (requests leave in issue order): the receive side
     // may now flood it with row reads without delaying these few words.
     compiler_barrier();
     if (lane == 0) device_store(state.receive_prefix_state, epoch | kPrefixRequested);
     compiler_barrier();
+    if (own_from_plan) {
+        // ... then the own words, out of device memory, once the plan is there.
+        if (!wait_for_plan(state, *state.queues, lane)) return false;
+        if (lane == me) unique = device_load(unique_address);
+#pragma unroll
+        for (int i = 0; i < kExpectedPerLane; ++i)
+            if (expected_address[i] && (lane + i * kWave) % ranks == me) expected_values[i] = device_load(expected_address[i]);
+#pragma unroll
+        for (int source = 0; source < kMaxRanks; ++source)
+            if (source == me && first_address[source]) first_counts[source] = device_load(first_address[source]);
+    }
     // Per-source unique counts -> source_offsets (lane = source).
     int inclusive = unique;
     PCIE_EP_PROFILE(if (__builtin_amdgcn_readfirstlane(inclusive) >= 0) profile.first(kProfilePrefixMailboxNs);)  // the first use of a mailbox word: the reads have returned
@@ -220,6 +283,7 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE
 #pragma unroll
         for (int source = 0; source < kMaxRanks; ++source) {
             if (begin == 0) counts[source] = first_counts[source];
+            else if (own_from_plan && source == me) counts[source] = expert < local ? device_load(state.plan_counts + ranks + me * local + expert) : 0;
             else counts[source] = (source < ranks && expert < local) ? host_field_load(mailbox_at(z, state.seg[source], me) + 1 + expert) : 0;
         }
         int running = 0;
@@ -265,23 +329,44 @@ __device__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE
 // A source may overwrite its count mailbox for the next epoch once this rank has
 // said so.  Every lane has its counts in registers by now (the loads above were
 // waited for, wave-wide), so the ACK needs no fence (advanced_layout.cuh:91-93).
-__device__ void acknowledge_counts(const DeviceState& state, int lane) {
+__device__ __forceinline__ void acknowledge_counts(const DeviceState& state, int lane) {
     const SegmentLayout& z = state.z;
     wait_memory_ops();
     if (lane < z.dims.num_ranks && lane != state.local_rank && lane != state.counts_ack_skip_source)
-        host_field_store(signal_at(state.seg[lane], z.counts_consumed_offset, state.local_rank), *state.epoch);
+        host_field_store(signal_at(state.seg[lane], z.counts_consumed_offset, state.local_rank), dispatch_epoch(state));
 }
+
+__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile));
 
 // One wavefront of the grid (the first RX control to get there) computes the
 // receive prefixes; nobody waits here.
-__device__ void elect_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
-    const uint64_t epoch = *state.epoch;
+__device__ __forceinline__ void elect_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
+    const uint64_t epoch = dispatch_epoch(state);
     int claimed = 0;
     if (lane == 0) {
         unsigned long long expected = 0;
         claimed = atomicCAS(reinterpret_cast<unsigned long long*>(state.receive_prefix_state), expected, epoch) == 0ull;
     }
     if (!broadcast_first(claimed)) return;
+    produce_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+}
+
+// With payload workgroups of their own, the control workgroups have wavefronts to
+// spare (a third one exists with three or more payload wavefronts per workgroup):
+// the receive prefixes are then produced by that one (wavefront 2 of
+// channel 0's workgroup) and no RX control is held up by them - the channel of an
+// elected RX control starts to receive a prefix computation late.
+__device__ __forceinline__ bool dedicated_prefix_producer(const DeviceState& state) { return state.worker_groups > 0 && state.tx_waves + state.rx_waves >= 3; }
+
+__device__ __forceinline__ void receive_prefix_role(const DeviceState& state, int lane) {
+    PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
+    if (lane == 0) device_store(state.receive_prefix_state, dispatch_epoch(state));
+    produce_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+    PCIE_EP_PROFILE(profile.save(state.profiling, profile_rows(state.z.dims.channels, state.worker_groups * (state.tx_waves + state.rx_waves)) - 1, lane);)
+}
+
+__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
+    const uint64_t epoch = dispatch_epoch(state);
     const bool success = compute_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
     // The results were written through; they are complete once this wavefront's
     // stores have been acknowledged.  Local consumers come first, the ACK to the
@@ -312,14 +397,14 @@ __device__ __forceinline__ int receive_prefix_verdict(const DeviceState& state, 
 // ---------------------------------------------------------------------------------------
 // TX control + guardian
 // ---------------------------------------------------------------------------------------
-__device__ void tx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
+__device__ __forceinline__ void tx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
     const SegmentLayout& z = state.z;
     const int channels = z.dims.channels, me = state.local_rank;
     const int endpoints = z.endpoints;  // destination ranks, then (relay mode) one relay endpoint per domain
     const int slots = z.dims.payload_slots;
     const int stride = (z.dims.max_tokens + channels - 1) / channels;
     char* own = state.seg[me];
-    const uint64_t epoch = *state.epoch;
+    const uint64_t epoch = dispatch_epoch(state);
     const uint64_t start = now_ticks();
     HealthCheck health(state, start, true, channel, channels);
     PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
@@ -332,7 +417,7 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
     int reserved[kMaxEndpoints];
 #pragma unroll
     for (int endpoint = 0; endpoint < kMaxEndpoints; ++endpoint) reserved[endpoint] = 0;
-    bool failed = false;
+    bool failed = !wait_for_plan(state, q, lane);
     int64_t stage_busy = 0, prepared_ahead = 0;
 
     for (int base = 0; base < candidates && !failed; base += kWave) {
@@ -504,13 +589,13 @@ __device__ void tx_control(const DeviceState& state, TransportQueues& q, int cha
 // ---------------------------------------------------------------------------------------
 // RX control
 // ---------------------------------------------------------------------------------------
-__device__ void rx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
+__device__ __forceinline__ void rx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, me = state.local_rank;
     const uint64_t begin = now_ticks();
-    const uint64_t epoch = *state.epoch;
+    const uint64_t epoch = dispatch_epoch(state);
     PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
-    elect_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+    if (!dedicated_prefix_producer(state)) elect_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
     // Polling does not wait for the prefixes: a descriptor entry is valid as soon as
     // its tag carries this epoch and the next ordinal, whatever the counts say, so
     // rows are requested from the first microseconds of the kernel on.  The counts
@@ -571,6 +656,18 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
             PCIE_EP_PROFILE(profile.add(kProfilePollMisses);)
             ++not_ready;
             backoff();
+            // Prologue in the same launch: no row can be handed out before the own counts
+            // are with the peers, and until then every poll here is a read on the host
+            // link in front of the acknowledgement those counts wait for.  After the
+            // first look, polling pauses until that point (bounded by the abort word,
+            // which the prologue and the guardians raise).
+            while (state.fused && !gate_open) {
+                int outcome = 0;
+                if (lane == 0) outcome = device_load(&q.plan_ready.value) == epoch_flag(epoch) ? 1 : (aborted(q) ? -1 : 0);
+                outcome = broadcast_first(outcome);
+                if (outcome) break;
+                __builtin_amdgcn_s_sleep(16);
+            }
             continue;
         }
         // Slot and token come from the peer (or its relay) and become the base of a
@@ -596,7 +693,10 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
         // queue behind megabytes of row reads.
         while (!gate_open) {
             int gate = 0;
-            if (lane == 0) gate = (device_load(state.receive_prefix_state) & kPrefixRequested) ? 1 : (aborted(q) ? -1 : 0);
+            // Prologue in the same launch: and not before the own counts are with the peers.
+            if (lane == 0)
+                gate = ((device_load(state.receive_prefix_state) & kPrefixRequested) && (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch)))
+                           ? 1 : (aborted(q) ? -1 : 0);
             gate = broadcast_first(gate);
             if (gate > 0) gate_open = true;
             else if (gate < 0 || receive_prefix_verdict(state, epoch, lane) < 0) {
@@ -679,8 +779,8 @@ __device__ void rx_control(const DeviceState& state, TransportQueues& q, int cha
 // layout) the local experts' alignment gaps.  Every wavefront of the local
 // workgroups claims items one at a time until none is left.
 template <bool kVector>
-__device__ void local_rows(const DeviceState& state, TransportQueues& q, int lane) {
-    const uint64_t epoch = *state.epoch;
+__device__ __forceinline__ void local_rows(const DeviceState& state, TransportQueues& q, int lane) {
+    const uint64_t epoch = dispatch_epoch(state);
     // Destination rows depend on the receive prefixes of this epoch.
     int ready = 0;
     if (lane == 0) {
@@ -693,6 +793,7 @@ __device__ void local_rows(const DeviceState& state, TransportQueues& q, int lan
         }
     }
     if (!broadcast_first(ready)) return;
+    if (!wait_for_plan(state, q, lane)) return;
     const bool padding = state.expand && state.fuse_expand && state.zero_padding;
     const int items = state.num_tokens + (padding ? state.z.local_experts : 0);
     while (true) {
@@ -715,7 +816,7 @@ __device__ void local_rows(const DeviceState& state, TransportQueues& q, int lan
 // Called by every role wavefront as its last act.  Everything the reduction
 // reads was written with device-scope stores or atomics, so waiting for this
 // wavefront's own operations is all the ordering the count needs.
-__device__ void finish_role(const DeviceState& state, TransportQueues& q, int lane, uint32_t roles) {
+__device__ __forceinline__ void finish_role(const DeviceState& state, TransportQueues& q, int lane, uint32_t roles) {
     wait_memory_ops();
     uint32_t earlier = 0;
     if (lane == 0) earlier = device_add(&q.finished.value, 1u);
@@ -723,30 +824,42 @@ __device__ void finish_role(const DeviceState& state, TransportQueues& q, int la
     // Last one out: column sums of the per-channel statistics and the span of
     // the channel timestamps.  Done after failures too (the reference launches
     // advanced_reduce_statistics unconditionally).
+    // The whole kernel waits for this wavefront: every word is requested before the
+    // first is used (lane l reads words l, l + 64, ...), and the sums and the span
+    // come out of lane shuffles - two round trips to memory, not one per channel.
     const int channels = state.z.dims.channels;
-    if (lane < kStatFields) {
-        int64_t sum = 0;
-        for (int channel = 0; channel < channels; ++channel) sum += device_load(state.channel_stats + channel * kStatFields + lane);
-        state.stats[lane] = sum;
+    constexpr int kStatWordsPerLane = kMaxChannels * kStatFields / kWave;
+    int64_t words[kStatWordsPerLane];
+#pragma unroll
+    for (int i = 0; i < kStatWordsPerLane; ++i) {
+        const int word = lane + i * kWave;
+        words[i] = word < channels * kStatFields ? device_load(state.channel_stats + word) : 0;
     }
-    if (lane == 0) {
-        int64_t start = 0, end = 0;
-        for (int channel = 0; channel < channels; ++channel) {
-            const int64_t begin = device_load(state.channel_timestamps_ns + channel * 2);
-            if (begin && (!start || begin < start)) start = begin;
-            const int64_t finish = device_load(state.channel_timestamps_ns + channel * 2 + 1);
-            if (finish > end) end = finish;
-        }
-        state.transport_timestamps_ns[0] = start;
-        state.transport_timestamps_ns[1] = end;
+    // Channel c's start and end stamps are words 2c and 2c + 1: lane l takes word l.
+    const int64_t stamp = lane < channels * 2 ? device_load(state.channel_timestamps_ns + lane) : 0;
+    // kStatFields divides 64: word w belongs to field w % kStatFields whatever i is.
+    int64_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kStatWordsPerLane; ++i) sum += words[i];
+    for (int offset = kStatFields; offset < kWave; offset <<= 1) sum += __shfl_xor(sum, offset);
+    if (lane < kStatFields) state.stats[lane] = sum;
+    // Even lanes hold start stamps (earliest non-zero wins), odd lanes end stamps (latest wins).
+    int64_t span = lane % 2 == 0 && stamp == 0 ? INT64_MAX : stamp;
+    for (int offset = 2; offset < kWave; offset <<= 1) {
+        const int64_t other = __shfl_xor(span, offset);
+        span = lane % 2 == 0 ? (other < span ? other : span) : (other > span ? other : span);
     }
+    if (lane == 0) state.transport_timestamps_ns[0] = span == INT64_MAX ? 0 : span;
+    if (lane == 1) state.transport_timestamps_ns[1] = span;
+    // Prologue inside this launch: every workgroup has read the epoch word by now.
+    if (lane == 0 && state.fused) *state.epoch = dispatch_epoch(state);
 }
 
 // ---------------------------------------------------------------------------------------
 // TX payload worker
 // ---------------------------------------------------------------------------------------
 template <bool kFp8, bool kVector>
-__device__ float tx_copy_row(const DeviceState& state, const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int lane) {
+__device__ __forceinline__ float tx_copy_row(const DeviceState& state, const uint16_t* input, __amdgpu_buffer_rsrc_t slot, int lane) {
     const int hidden = state.z.dims.hidden;
     if constexpr (kFp8) return quantize_row<kVector>(input, HostCodes{slot}, hidden, lane);
     copy_row_to_host<kVector>(input, slot, hidden, lane);
@@ -761,7 +874,7 @@ struct WorkerCounters {
 // Moves the own token of transmit ticket `ticket_index` (already marked ready)
 // into its host slot and publishes it.  Returns false when the wavefront must stop.
 template <bool kFp8, bool kVector>
-__device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, const Deadline& deadline,
+__device__ __forceinline__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, const Deadline& deadline,
                        WorkerCounters& counters PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, topk = z.dims.topk, me = state.local_rank;
@@ -769,7 +882,7 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
     const int slots = z.dims.payload_slots, descriptors = z.dims.descriptor_slots;
     const int stride = (z.dims.max_tokens + z.dims.channels - 1) / z.dims.channels;
     char* own = state.seg[me];
-    const uint64_t epoch = *state.epoch;
+    const uint64_t epoch = dispatch_epoch(state);
     const int meta_dwords = z.meta_bytes / 4;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.tx, sizeof(q.tx));
     {
@@ -869,12 +982,12 @@ __device__ bool tx_row(const DeviceState& state, TransportQueues& q, uint32_t* s
 // host slot and stores it to its destination rows.  Returns false when the
 // wavefront must stop.
 template <bool kFp8, bool kVector>
-__device__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters,
+__device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters,
                        bool& prefixes_known PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
-    const uint64_t epoch = *state.epoch;
+    const uint64_t epoch = dispatch_epoch(state);
     const bool scatter = state.expand && state.fuse_expand;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
     {
@@ -1144,8 +1257,8 @@ constexpr int kMinTxWaves = 16;
 constexpr uint64_t kIdleCrossoverUs = 30;
 
 template <bool kFp8, bool kVector>
-__device__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int order, int waves) {
-    const uint64_t epoch = *state.epoch;
+__device__ __forceinline__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int order, int waves) {
+    const uint64_t epoch = dispatch_epoch(state);
     Deadline deadline(now_ticks());
     WorkerCounters counters;
     PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz); uint64_t idle_begin = 0; int rows_moved = 0;)
@@ -1236,11 +1349,20 @@ __device__ void payload_worker(const DeviceState& state, TransportQueues& q, uin
 // no payload workgroups configured the control workgroups carry the payload
 // wavefronts themselves.
 template <bool kFp8, bool kVector>
-__global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceState state) {
+__global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceState launch_state) {
+    // The launch argument is read where it lies, in the kernel-argument segment:
+    // every field is then a scalar load from constant memory and every pointer in
+    // it a global pointer.  A by-value copy would be a private object of 1 KB that
+    // each role reads back through scratch loads, with generic pointers in it.
+#if defined(__HIP_DEVICE_COMPILE__)
+    const DeviceState& state = *reinterpret_cast<const DeviceState*>(__builtin_amdgcn_kernarg_segment_ptr());
+#else
+    const DeviceState& state = launch_state;  // the host pass only parses the kernel
+#endif
     __shared__ WaveScratch lds;
+    extern __shared__ __align__(16) unsigned char prologue_lds[];  // sized by the launcher when the prologue rides in this launch
     const int channels = state.z.dims.channels;
-    if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) return;
-    const int block = blockIdx.x;
+    int block = blockIdx.x;
     int wave = threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
     uint32_t* scratch = lds.words[wave];
@@ -1248,18 +1370,47 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
     const int payload_waves = state.tx_waves + state.rx_waves;
     const int payload_groups = state.worker_groups > 0 ? state.worker_groups : 0;
     const int waves_per_group = int(blockDim.x) / kWave;
-    const uint32_t roles = uint32_t(2 * channels + (payload_groups ? payload_groups : channels) * payload_waves + state.local_groups * waves_per_group);
+    const int prologue_groups = fused_prologue_groups(state);
+    // Role wavefronts of the launch: controls, payload and local-bypass wavefronts, the producer of the receive
+    // prefixes where it is a wavefront of its own, one per prologue workgroup and a second one for the epoch begin.
+    const uint32_t roles = uint32_t(2 * channels + (payload_groups ? payload_groups : channels) * payload_waves + state.local_groups * waves_per_group +
+                                    (dedicated_prefix_producer(state) ? 1 : 0) + prologue_groups + (prologue_groups ? 1 : 0));
+    bool begun = true;
+    if (state.fused) {
+        // The prologue's workgroups carry the lowest indices: they are started first.
+        // Workgroup 0 begins the epoch, the ones after it lay out one chunk of tokens each.
+        if (block < prologue_groups) {
+            if (block == 0) {
+                if (wave >= 2) return;
+                epoch_begin_role(state, wave, lane);
+                return finish_role(state, q, lane, roles);
+            }
+            prologue_chunk<8, true>(state, prologue_lds, waves_per_group, state.prologue_chunks, block - 1);
+            if (wave == 0) finish_role(state, q, lane, roles);
+            return;
+        }
+        block -= prologue_groups;
+        begun = __syncthreads_or(threadIdx.x == 0 ? int(wait_for_begin(state, q)) : 0) != 0;
+    } else if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) {
+        return;  // the prologue kernel in front of this one failed
+    }
     if (block >= channels + payload_groups) {
-        local_rows<kVector>(state, q, lane);
+        if (begun) local_rows<kVector>(state, q, lane);
         return finish_role(state, q, lane, roles);
     }
     if (block < channels) {
         if (wave < 2) {
-            if (wave == 0) tx_control(state, q, block, lane);
-            else rx_control(state, q, block, lane);
+            if (begun) {
+                if (wave == 0) tx_control(state, q, block, lane);
+                else rx_control(state, q, block, lane);
+            }
             return finish_role(state, q, lane, roles);
         }
-        if (payload_groups) return;
+        if (payload_groups) {
+            if (block != 0 || wave != 2 || !dedicated_prefix_producer(state)) return;
+            if (begun) receive_prefix_role(state, lane);
+            return finish_role(state, q, lane, roles);
+        }
         wave -= 2;
     }
     if (wave >= payload_waves) return;
@@ -1267,7 +1418,7 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
     // direction's share is spread over the workgroups before it doubles up in one.
     const int groups = payload_groups ? payload_groups : channels;
     const int group = payload_groups ? block - channels : block;
-    payload_worker<kFp8, kVector>(state, q, scratch, lane, wave * groups + group, groups * payload_waves);
+    if (begun) payload_worker<kFp8, kVector>(state, q, scratch, lane, wave * groups + group, groups * payload_waves);
     finish_role(state, q, lane, roles);
     // Every role loop has an explicit completion, abort or timeout exit and no
     // workgroup barrier follows the entry verdict.
@@ -1288,23 +1439,32 @@ hipError_t transport_workgroups_per_unit(const DeviceState& state, int* per_unit
     if (threads > kTransportMaxThreads) return hipErrorInvalidValue;
     const bool fp8 = state.z.dims.wire_fp8 != 0;
     const bool vector = fp8 ? state.z.dims.hidden % 16 == 0 : state.z.dims.hidden % 8 == 0;
-    if (fp8 && vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, true>, threads, 0);
-    if (fp8) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, false>, threads, 0);
-    if (vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, true>, threads, 0);
-    return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, false>, threads, 0);
+    const size_t lds = state.fused ? prologue_lds_bytes(state.z, threads / kWave) : 0;
+    if (fp8 && vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, true>, threads, lds);
+    if (fp8) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<true, false>, threads, lds);
+    if (vector) return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, true>, threads, lds);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_unit, transport_kernel<false, false>, threads, lds);
 }
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
-    const dim3 grid(state.z.dims.channels + (state.worker_groups > 0 ? state.worker_groups : 0) + state.local_groups), block(transport_threads(state));
+    const int prologue_groups = fused_prologue_groups(state);
+    const dim3 grid(prologue_groups + state.z.dims.channels + (state.worker_groups > 0 ? state.worker_groups : 0) + state.local_groups),
+        block(transport_threads(state));
     if (int(block.x) > kTransportMaxThreads) return hipErrorInvalidValue;
+    size_t dynamic_lds = 0;
+    if (state.fused) {
+        // The prologue's chunks are the workgroup's own wavefronts; the conditions are those of fused_prologue_fits().
+        if (!fused_prologue_fits(state.z, int(block.x), state.z.dims.max_tokens)) return hipErrorInvalidValue;
+        dynamic_lds = prologue_lds_bytes(state.z, int(block.x) / kWave);
+    }
     const bool fp8 = state.z.dims.wire_fp8 != 0;
     // BF16 rows need 16-byte granularity on both sides; FP8 additionally needs
     // whole 16-code vectors on the wire.
     const bool vector = fp8 ? state.z.dims.hidden % 16 == 0 : state.z.dims.hidden % 8 == 0;
-    if (fp8 && vector) hipLaunchKernelGGL((transport_kernel<true, true>), grid, block, 0, stream, state);
-    else if (fp8) hipLaunchKernelGGL((transport_kernel<true, false>), grid, block, 0, stream, state);
-    else if (vector) hipLaunchKernelGGL((transport_kernel<false, true>), grid, block, 0, stream, state);
-    else hipLaunchKernelGGL((transport_kernel<false, false>), grid, block, 0, stream, state);
+    if (fp8 && vector) hipLaunchKernelGGL((transport_kernel<true, true>), grid, block, dynamic_lds, stream, state);
+    else if (fp8) hipLaunchKernelGGL((transport_kernel<true, false>), grid, block, dynamic_lds, stream, state);
+    else if (vector) hipLaunchKernelGGL((transport_kernel<false, true>), grid, block, dynamic_lds, stream, state);
+    else hipLaunchKernelGGL((transport_kernel<false, false>), grid, block, dynamic_lds, stream, state);
     return hipGetLastError();
 }
 

@@ -25,8 +25,8 @@ class Config(C.Structure):
         "num_ranks", "local_rank", "max_tokens", "hidden", "topk", "num_experts", "channels", "payload_slots",
         "descriptor_slots", "wire_fp8", "timeout_ms", "fuse_receive_expand", "tx_waves", "rx_waves", "peer_threads",
         "staging_numa_node", "device", "worker_groups", "receive_expand_mode", "numa_mode", "replica_slots",
-        "relay_workers_per_numa", "relay_cpu_count")] + [
-        ("reserved", C.c_int32 * 5), ("rank_numa_nodes", C.c_int32 * 16), ("relay_cpus", C.c_int32 * 64), ("relay_delay_ns", C.c_uint64)]
+        "relay_workers_per_numa", "relay_cpu_count", "split_launch")] + [
+        ("reserved", C.c_int32 * 4), ("rank_numa_nodes", C.c_int32 * 16), ("relay_cpus", C.c_int32 * 64), ("relay_delay_ns", C.c_uint64)]
 
 
 class Sizes(C.Structure):

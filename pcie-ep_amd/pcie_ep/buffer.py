@@ -143,6 +143,7 @@ class HostStagedEPBuffer:
         worker_groups: int = 0,
         rank_numa_nodes: Optional[Tuple[int, ...]] = None,
         comm_stream_cus: int = 0,
+        split_launch: bool = False,
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
@@ -169,6 +170,11 @@ class HostStagedEPBuffer:
         must hold every control and payload workgroup of a dispatch at once (checked
         here, ``ValueError`` otherwise: 80 workgroups at the defaults); 32 units
         carry the dispatch at full link rate.
+        ``split_launch=True`` runs the prologue (epoch begin, layout, count
+        publication) as a kernel of its own in front of the transport kernel; by
+        default it rides in the transport kernel's launch wherever it fits (top-k up
+        to 8, default launch shape), so that a dispatch is one launch and the receive
+        side starts while the layout is computed.
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -216,7 +222,7 @@ class HostStagedEPBuffer:
         self.runtime = NativeRuntime(rank, num_ranks, num_max_tokens_per_rank, hidden, num_topk, num_experts, self.config,
                                      self.device, peer_threads=threads, staging_numa_node=staging_numa_node,
                                      tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups,
-                                     rank_numa_nodes=rank_numa_nodes)
+                                     rank_numa_nodes=rank_numa_nodes, split_launch=split_launch)
         if comm_stream_cus:
             # Control and payload workgroups wait for each other through device memory:
             # the masked units must hold all of them at once, or every dispatch would

@@ -7,7 +7,9 @@ role wavefront, written once when the role ends.  Build the variant with
 ``PCIE_EP_PROFILING=1`` before importing ``pcie_ep``.
 
 Rows: TX control ``[0, C)``, RX control ``[C, 2C)``, payload wavefronts
-``[2C, 2C + W)``, prologue leader ``[2C + W]``.  Stamps (``*_ns``) are
+``[2C, 2C + W)``, prologue leader ``[2C + W]``, epoch begin ``[2C + W + 1]``, producer of the
+receive prefixes ``[2C + W + 2]`` (the last two hold records only where those are
+roles of their own; ``read`` folds their stamps into the leader's and RX control 0's).  Stamps (``*_ns``) are
 nanoseconds of the device wall clock, sums are accumulated nanoseconds; a zero
 stamp means the event did not happen.  Intervals of different roles overlap.
 """
@@ -27,7 +29,8 @@ CONTROL = COMMON + ("first_ticket_ns", "last_ticket_ns", "workers_done_ns", "dra
                     "prefix_counts_ready_ns", "prefix_mailbox_ns", "prefix_published_ns")
 WORKER = COMMON + ("first_claim_ns", "last_row_ns", "tx_rows", "rx_rows", "sampled_tx_rows", "sampled_rx_rows", "ticket_wait_sum",
                    "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum")
-PROLOGUE = COMMON + ("layout_ns", "totals_ns", "verdict_ns", "mailbox_free_ns", "mailbox_acked_ns", "counts_ready_ns")
+PROLOGUE = COMMON + ("layout_ns", "totals_ns", "verdict_ns", "mailbox_free_ns", "mailbox_acked_ns", "counts_ready_ns",
+                     "begun_ns", "routes_ns", "masks_ns", "chunk_totals_ns", "plan_ready_ns")
 
 
 def read(runtime) -> Dict[str, np.ndarray]:
@@ -41,7 +44,21 @@ def read(runtime) -> Dict[str, np.ndarray]:
     table = np.zeros((rows.value, fields.value), dtype=np.int64)
     _native.check(lib.pcie_ep_profile_read(runtime.handle, table.ctypes.data_as(C.POINTER(C.c_int64))), invalid=RuntimeError)
     c, w = channels.value, wavefronts.value
-    return {"tx_control": table[:c], "rx_control": table[c : 2 * c], "workers": table[2 * c : 2 * c + w], "prologue": table[2 * c + w]}
+    prologue = table[2 * c + w].copy()
+    begin = table[2 * c + w + 1]
+    # The epoch begin keeps a record of its own where it is a workgroup of its own
+    # (prologue inside the transport launch); its stamps are folded into the leader's.
+    if begin[0]:
+        for name in ("begun_ns", "verdict_ns", "mailbox_free_ns"):
+            prologue[PROLOGUE.index(name)] = begin[PROLOGUE.index(name)]
+    # Likewise the producer of the receive prefixes: its stamps are folded into RX control 0's.
+    rx_control = table[c : 2 * c].copy()
+    producer = table[2 * c + w + 2]
+    if producer[0]:
+        for name in ("prefix_enter_ns", "prefix_counts_ready_ns", "prefix_mailbox_ns", "prefix_published_ns"):
+            rx_control[0, CONTROL.index(name)] = producer[CONTROL.index(name)]
+    return {"tx_control": table[:c], "rx_control": rx_control, "workers": table[2 * c : 2 * c + w], "prologue": prologue,
+            "epoch_begin": begin, "prefix_producer": producer}
 
 
 def _col(rows: np.ndarray, names, name: str) -> np.ndarray:

@@ -73,7 +73,7 @@ class NativeRuntime:
 
     def __init__(self, rank: int, world: int, max_tokens: int, hidden: int, topk: int, experts: int, config: HostStagedConfig,
                  device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0,
-                 worker_groups: int = 0, rank_numa_nodes: Optional[tuple] = None) -> None:
+                 worker_groups: int = 0, rank_numa_nodes: Optional[tuple] = None, split_launch: bool = False) -> None:
         self._lib = _native.library()
         self.config = config
         self.device = torch.device("cuda", device)
@@ -88,6 +88,7 @@ class NativeRuntime:
             receive_expand_mode=("pipelined", "vectorized", "scalar").index(config.receive_expand_mode),
             numa_mode=int(config.numa_mode == "relay"), replica_slots=config.replica_slots,
             relay_workers_per_numa=config.relay_workers_per_numa, relay_cpu_count=len(config.relay_cpu_affinity),
+            split_launch=int(split_launch),
         )
         if len(config.relay_cpu_affinity) > 64:
             raise ValueError("relay_cpu_affinity holds more than 64 CPUs")
