@@ -189,6 +189,54 @@ __device__ __forceinline__ uint64_t dispatch_epoch(const DeviceState& state) { r
 __host__ __device__ __forceinline__ int fused_prologue_groups(const DeviceState& state) {
     return state.fused ? 1 + (state.prologue_chunks > 1 ? state.prologue_chunks : 1) : 0;
 }
+// Which workgroup runs where.  Consecutive workgroup ids go to consecutive XCDs (eight of them), and everything a
+// wavefront sends to memory passes through its XCD's L2 queues, where a host read stays for as long as the host link
+// needs for all the bytes requested before it.  A control path that shares an XCD with payload wavefronts therefore
+// sees every one of its device-memory operations take that long too - tickets, prefixes and flags arrive tens of
+// microseconds late as soon as rows are in flight.  With payload workgroups of their own, the launch therefore
+// gives the first kControlXcds XCDs to the control class (epoch begin, layout chunks, channel controls) and the
+// other six to the payload class (payload and local-bypass workgroups): workgroup id = row * 8 + XCD; ids that fall
+// behind the end of their class are fillers that end at once.  Without payload workgroups the ids are linear.
+constexpr int kXcds = 8, kControlXcds = 2;
+// Channel control workgroups: one per channel (both of its controls) without payload workgroups of their own;
+// with them, one per direction and pair of channels.
+__host__ __device__ __forceinline__ int control_groups(const DeviceState& state) {
+    const int channels = state.z.dims.channels;
+    return state.worker_groups > 0 ? (channels + 1) / 2 * 2 : channels;
+}
+struct TransportGrid {
+    int control_class;   // epoch begin + layout chunks (prologue in this launch) + channel control workgroups
+    int payload_class;   // payload workgroups + local-bypass workgroups
+    int rows;            // 0: linear ids (control class first)
+    int blocks;
+};
+__host__ __device__ __forceinline__ TransportGrid transport_grid(const DeviceState& state) {
+    TransportGrid grid;
+    const int payload_groups = state.worker_groups > 0 ? state.worker_groups : 0;
+    grid.control_class = fused_prologue_groups(state) + control_groups(state);
+    grid.payload_class = payload_groups + state.local_groups;
+    if (!payload_groups) {
+        grid.rows = 0;
+        grid.blocks = grid.control_class + grid.payload_class;
+        return grid;
+    }
+    const int control_rows = (grid.control_class + kControlXcds - 1) / kControlXcds;
+    const int payload_rows = (grid.payload_class + kXcds - kControlXcds - 1) / (kXcds - kControlXcds);
+    grid.rows = control_rows > payload_rows ? control_rows : payload_rows;
+    grid.blocks = grid.rows * kXcds;
+    return grid;
+}
+// Logical index of a workgroup id (control class first, then the payload class), -1 for a filler.
+__host__ __device__ __forceinline__ int transport_block(const TransportGrid& grid, int id) {
+    if (!grid.rows) return id;
+    const int xcd = id % kXcds, row = id / kXcds;
+    if (xcd < kControlXcds) {
+        const int index = row * kControlXcds + xcd;
+        return index < grid.control_class ? index : -1;
+    }
+    const int index = row * (kXcds - kControlXcds) + xcd - kControlXcds;
+    return index < grid.payload_class ? grid.control_class + index : -1;
+}
 // 32-bit value an epoch-tagged flag word carries (epochs stay below 2^32; the one beyond, which only ends in error 20, still gets a value of its own).
 __device__ __forceinline__ uint32_t epoch_flag(uint64_t epoch) { return uint32_t(epoch) + uint32_t(epoch >> 32) * 0x9E3779B9u; }
 
@@ -212,7 +260,7 @@ enum ProfileField : int {
     kProfilePollSum,             // time inside those polls
     kProfileHealthScans, kProfileHealthSum,
     kProfileCountsKnownNs,       // RX control: receive prefixes seen
-    kProfileGateOpenNs,          // RX control: first ticket allowed out (count mailbox reads are on the link)
+    kProfileControlSpare,        // (not used)
     // receive-prefix producer (in the record of the RX control that was elected)
     kProfilePrefixEnterNs = 16, kProfilePrefixCountsReadyNs, kProfilePrefixMailboxNs, kProfilePrefixPublishedNs,
     // ---- payload wavefronts (rows [2C, 2C + W)); field 3 = rows moved ----
@@ -227,6 +275,7 @@ enum ProfileField : int {
     kProfileRxRequestSum,        // sampled: row loads issued -> metadata and payload returned
     kProfileRxPrefixWaitSum,     // sampled: waiting for the receive prefixes (first rows only)
     kProfileRxScatterSum,        // sampled: row loads issued -> destination rows' stores issued
+    kProfileGateOpenNs,          // first received row: the gate in front of the row requests seen open
 };
 // Record of the prologue's leader workgroup (thread 0), stored behind the payload wavefronts' records.
 enum PrologueProfileField : int {
@@ -401,6 +450,14 @@ __device__ __forceinline__ T device_load(const T* address) {
 template <typename T>
 __device__ __forceinline__ void device_store(T* address, T value) {
     __hip_atomic_store(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// The same for an address the compiler cannot trace back to a kernel argument
+// (one rebuilt from lane shuffles, say): stating the global address space keeps
+// the access a global load instead of a flat one, which would be waited for on
+// both memory counters before anything else is issued.
+__device__ __forceinline__ int32_t device_load_global(const int32_t* address) {
+    typedef const int32_t __attribute__((address_space(1))) * GlobalWord;
+    return __hip_atomic_load((GlobalWord)address, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint32_t device_add(uint32_t* address, uint32_t value) {
     return __hip_atomic_fetch_add(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

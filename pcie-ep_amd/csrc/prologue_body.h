@@ -243,18 +243,21 @@ __device__ __forceinline__ bool begin_epoch(const DeviceState& state, uint64_t t
     return !begin_failed;
 }
 
-// Inside the transport launch the epoch begins in a workgroup of its own, as two
+// Inside the transport launch the epoch begins in a workgroup of its own, as
 // independent wavefronts (memory operations of a wavefront complete in order, so
 // one that has asked for host words cannot learn that its stores have arrived
 // before those words are back):
 //  * wavefront 0 clears (written through) and announces `begun`, which every
 //    other role of the launch waits for before it touches the queues or records
 //    anything;
-//  * wavefront 1 reads the abort words and waits for the count mailbox; on
-//    success it announces `verdict`, which the layout's leader waits for before it
-//    stores the counts, otherwise it records the error (after `begun`) and raises
-//    the launch's abort word.
-__device__ __forceinline__ void epoch_begin_role(const DeviceState& state, int wave, int lane) {
+//  * the other wavefronts share the abort words between them (the round trip of a
+//    few hundred scattered host words is shorter from several wavefronts); the
+//    helpers hand their findings to wavefront 1 through LDS, which also waits for
+//    the count mailbox; on success it announces `verdict`, which the layout's
+//    leader waits for before it stores the counts, otherwise it records the error
+//    (after `begun`) and raises the launch's abort word.
+// Wavefronts 0 and 1 are roles of the launch (they call finish_role), the helpers are not.
+__device__ __forceinline__ void epoch_begin_role(const DeviceState& state, int wave, int lane, int waves, int* findings) {
     const SegmentLayout& z = state.z;
     TransportQueues& q = *state.queues;
     char* own = state.seg[state.local_rank];
@@ -269,9 +272,22 @@ __device__ __forceinline__ void epoch_begin_role(const DeviceState& state, int w
                         if (lane == 0 && state.profiling) state.profiling[size_t(profile_row) * kProfileFields + kPrologueBegunNs] = int64_t(profile.values[kPrologueBegunNs]);)
         return;
     }
+    // findings[w]: 0 until reader w (1 .. waves - 1) has looked at its words, then 1 (none set) or 2.
+    const int readers = waves - 1;
+    if (wave > 1) {
+        const bool set = __any(read_abort_words(state, (wave - 1) * kWave + lane, readers * kWave));
+        if (lane == 0) lds_store(findings + wave, set ? 2 : 1);
+        return;
+    }
     uint64_t consumed_word = tag - 1;
     if (tag > 1 && lane < z.dims.num_ranks && lane != state.local_rank) consumed_word = host_load(signal_at(own, z.counts_consumed_offset, lane));
-    const bool any_abort = __any(read_abort_words(state, lane, kWave));
+    bool any_abort = __any(read_abort_words(state, lane, readers * kWave));
+    for (int helper = 2; helper < waves; ++helper) {
+        int finding = 0;
+        // The helpers end by themselves after one round trip over the host link.
+        while (!(finding = broadcast_first(lds_load(findings + helper)))) backoff();
+        any_abort |= finding == 2;
+    }
     PCIE_EP_PROFILE(profile.first(kPrologueVerdictNs);)
     int code = 0;
     if (tag >= 0x100000000ull) code = kErrEpochExhausted;

@@ -454,6 +454,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     rt->worker_groups = shape.worker_groups;
     {
         DeviceState probe{};
+        probe.z = rt->z;
         probe.tx_waves = rt->tx_waves;
         probe.rx_waves = rt->rx_waves;
         probe.worker_groups = rt->worker_groups;
@@ -461,7 +462,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         // (epoch begin, prologue chunks of a full batch, control, payload and local-bypass workgroups) is resident at once.
         const int block_threads = transport_threads(probe);
         rt->fused = !config->split_launch && fused_prologue_fits(rt->z, block_threads, dims.max_tokens) &&
-                    1 + prologue_chunks(rt->z, dims.max_tokens, block_threads / kWave) + dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0) + 32 <= 256;
+                    1 + prologue_chunks(rt->z, dims.max_tokens, block_threads / kWave) + control_groups(probe) + (rt->worker_groups > 0 ? rt->worker_groups : 0) + 32 <= 256;
     }
 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers
@@ -666,7 +667,7 @@ int pcie_ep_transport_residency(pcie_ep_runtime* rt, int32_t compute_units, int3
     HIP_TRY(transport_workgroups_per_unit(probe, &per_unit));
     // The control and payload workgroups wait for each other through device memory
     // and must run together; the local-bypass workgroups behind them may start late.
-    *needed = rt->z.dims.channels + (rt->worker_groups > 0 ? rt->worker_groups : 0) +
+    *needed = control_groups(probe) + (rt->worker_groups > 0 ? rt->worker_groups : 0) +
               (rt->fused ? 1 + std::max(1, prologue_chunks(rt->z, rt->z.dims.max_tokens, rt->tx_waves + rt->rx_waves)) : 0);
     *resident = per_unit * units;
     return 0;

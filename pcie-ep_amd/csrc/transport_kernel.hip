@@ -196,7 +196,7 @@ __device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& stat
     // The first look at every source's counts_ready is requested now; its value is
     // used after the address arithmetic below, which so runs inside its round trip.
     uint64_t first_look = 0;
-    if (lane < ranks && !(own_from_plan && lane == me)) first_look = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
+    if (lane < ranks && !(own_from_plan && lane == me)) first_look = host_load_global(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
     const auto segment_of = [&](int rank) {
         const uint64_t bits = reinterpret_cast<uint64_t>(lane_segment);
         return reinterpret_cast<char*>(uint64_t(uint32_t(__shfl(int(uint32_t(bits)), rank))) | uint64_t(uint32_t(__shfl(int(uint32_t(bits >> 32)), rank))) << 32);
@@ -224,7 +224,7 @@ __device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& stat
     bool ready = lane >= ranks || (own_from_plan && lane == me) || first_look == epoch;
     while (true) {
         if (__all(ready)) break;
-        if (!ready) ready = host_load(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset)) == epoch;
+        if (!ready) ready = host_load_global(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset)) == epoch;
         if (__all(ready)) break;
         if (health.poll(state, lane)) {
             if (lane == 0) record_error(state, kErrCountsReadyWait);
@@ -256,13 +256,13 @@ __device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& stat
     if (own_from_plan) {
         // ... then the own words, out of device memory, once the plan is there.
         if (!wait_for_plan(state, *state.queues, lane)) return false;
-        if (lane == me) unique = device_load(unique_address);
+        if (lane == me) unique = device_load_global(unique_address);
 #pragma unroll
         for (int i = 0; i < kExpectedPerLane; ++i)
-            if (expected_address[i] && (lane + i * kWave) % ranks == me) expected_values[i] = device_load(expected_address[i]);
+            if (expected_address[i] && (lane + i * kWave) % ranks == me) expected_values[i] = device_load_global(expected_address[i]);
 #pragma unroll
         for (int source = 0; source < kMaxRanks; ++source)
-            if (source == me && first_address[source]) first_counts[source] = device_load(first_address[source]);
+            if (source == me && first_address[source]) first_counts[source] = device_load_global(first_address[source]);
     }
     // Per-source unique counts -> source_offsets (lane = source).
     int inclusive = unique;
@@ -608,7 +608,7 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
     const bool replica = member && reads_replica(z.dims, source, me);
     const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
     int expected = member ? 0x7FFFFFFF : 0, total = 0x7FFFFFFF;
-    bool counts_known = false, prefix_failed = false, gate_open = false;
+    bool counts_known = false, prefix_failed = false;
     const uint64_t below = lanes_below(lane);
     const uint64_t group_mask = (1ull << lookahead) - 1ull;
     const __amdgpu_buffer_rsrc_t ring = device_resource(q.rx, sizeof(q.rx));
@@ -656,18 +656,6 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
             PCIE_EP_PROFILE(profile.add(kProfilePollMisses);)
             ++not_ready;
             backoff();
-            // Prologue in the same launch: no row can be handed out before the own counts
-            // are with the peers, and until then every poll here is a read on the host
-            // link in front of the acknowledgement those counts wait for.  After the
-            // first look, polling pauses until that point (bounded by the abort word,
-            // which the prologue and the guardians raise).
-            while (state.fused && !gate_open) {
-                int outcome = 0;
-                if (lane == 0) outcome = device_load(&q.plan_ready.value) == epoch_flag(epoch) ? 1 : (aborted(q) ? -1 : 0);
-                outcome = broadcast_first(outcome);
-                if (outcome) break;
-                __builtin_amdgcn_s_sleep(16);
-            }
             continue;
         }
         // Slot and token come from the peer (or its relay) and become the base of a
@@ -687,25 +675,6 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
                 break;
             }
         }
-        // The descriptors are polled from the start (a few dozen bytes per source),
-        // but no row is handed out before the producer of the prefixes has requested
-        // the count mailboxes: a few hundred bytes that everything waits for must not
-        // queue behind megabytes of row reads.
-        while (!gate_open) {
-            int gate = 0;
-            // Prologue in the same launch: and not before the own counts are with the peers.
-            if (lane == 0)
-                gate = ((device_load(state.receive_prefix_state) & kPrefixRequested) && (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch)))
-                           ? 1 : (aborted(q) ? -1 : 0);
-            gate = broadcast_first(gate);
-            if (gate > 0) gate_open = true;
-            else if (gate < 0 || receive_prefix_verdict(state, epoch, lane) < 0) {
-                prefix_failed = true;
-                break;
-            } else backoff();
-        }
-        if (prefix_failed) break;
-        PCIE_EP_PROFILE(profile.first(kProfileGateOpenNs);)
         const int ticket_index = reserve_tickets(q.rx_tail, __popcll(accepted), lane) + __popcll(accepted & below);
         const int slot = int(published[2]), token = int(published[3]);
         const uint64_t payload_sequence = sequence(epoch, token);
@@ -789,7 +758,7 @@ __device__ __forceinline__ void local_rows(const DeviceState& state, TransportQu
             if (value == epoch) { ready = 1; break; }
             // The wavefront that computes the prefixes owns the timeout.
             if (value == kPrefixFailed || aborted(q) || load_error_code(state)) break;
-            backoff();
+            __builtin_amdgcn_s_sleep(48);
         }
     }
     if (!broadcast_first(ready)) return;
@@ -983,7 +952,7 @@ __device__ __forceinline__ bool tx_row(const DeviceState& state, TransportQueues
 // wavefront must stop.
 template <bool kFp8, bool kVector>
 __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int ticket_index, WorkerCounters& counters,
-                       bool& prefixes_known PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
+                       const Deadline& deadline, bool& gate_open, bool& prefixes_known PCIE_EP_PROFILE(, RoleProfile& profile, bool sampled)) {
     const SegmentLayout& z = state.z;
     const int topk = z.dims.topk, me = state.local_rank, local = z.local_experts;
     const int hidden = z.dims.hidden;
@@ -1008,6 +977,30 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
         const __amdgpu_buffer_rsrc_t payload = host_resource(slot_base, uint32_t(z.payload_bytes));
         const __amdgpu_buffer_rsrc_t slot_meta = host_resource(slot_base + z.meta_offset, uint32_t(z.meta_bytes));
         if (lane == kWave - 1) test_delay(state.rx_delay);
+        // Tickets are handed out from the first descriptor on, but no row is requested
+        // before the producer of the prefixes has put its reads of the count mailboxes
+        // on the link (a few hundred bytes that everything waits for must not queue
+        // behind megabytes of row reads) nor, with the prologue in the same launch,
+        // before the own counts are with the peers (their acknowledgement would).
+        // The wavefront waits here with its ticket read and its addresses computed:
+        // the requests leave the moment the gate opens.
+        while (!gate_open) {
+            int gate = 0;
+            if (lane == 0) {
+                if ((device_load(state.receive_prefix_state) & kPrefixRequested) && (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch))) gate = 1;
+                else if (aborted(q) || device_load(state.receive_prefix_state + 1) == kPrefixFailed) gate = -1;
+                else if (deadline.expired(state)) {
+                    record_error(state, kErrRingProgressWait);
+                    raise_abort(q);
+                    gate = -1;
+                }
+            }
+            gate = broadcast_first(gate);
+            if (gate < 0) return false;
+            if (gate > 0) gate_open = true;
+            else __builtin_amdgcn_s_sleep(24);
+        }
+        PCIE_EP_PROFILE(profile.first(kProfileGateOpenNs);)
         // Column 0 of the receive/expand diagnostic: this row's host read starts
         // while an earlier row of the channel has not finished its scatter (the
         // conservative proof point of fused_receive.cuh:216-225; a count, not a time).
@@ -1058,7 +1051,9 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
             const int verdict = receive_prefix_verdict(state, epoch, lane);
             if (verdict < 0 || broadcast_first(aborted(q) ? 1 : 0)) return false;
             if (verdict > 0) prefixes_known = true;
-            else backoff();
+            // The row itself is microseconds away: a slow poll costs nothing, and a couple of hundred
+            // wavefronts polling fast would slow down the very stores of the prefixes they wait for.
+            else __builtin_amdgcn_s_sleep(48);
         }
 
         PCIE_EP_PROFILE(if (sampled) profile.add(kProfileRxPrefixWaitSum, profile.now() - prefix_begin);)
@@ -1255,6 +1250,7 @@ constexpr int64_t kTxWeight = 9, kRxWeight = 4;
 constexpr int64_t kTxLeadBytes = 24 << 20;
 constexpr int kMinTxWaves = 16;
 constexpr uint64_t kIdleCrossoverUs = 30;
+constexpr int kPreGateRows = 16;
 
 template <bool kFp8, bool kVector>
 __device__ __forceinline__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int order, int waves) {
@@ -1262,18 +1258,35 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
     Deadline deadline(now_ticks());
     WorkerCounters counters;
     PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz); uint64_t idle_begin = 0; int rows_moved = 0;)
-    bool prefixes_known = false;
+    bool prefixes_known = false, gate_open = false;
     const int lead = int(kTxLeadBytes / int64_t(state.z.meta_offset + state.z.meta_bytes));
     uint64_t idle_since = 0;  // 0: the last look found work
     while (true) {
         // 0: nothing to do now, 1: transmit, 2: receive, -1: both directions are finished or the kernel aborts.
         int choice = 0;
+        int gate_seen = gate_open ? 1 : 0;
         if (lane == 0) {
             if (aborted(q)) choice = -1;
             else {
                 const int tx_head = int(device_load(&q.tx_head.value)), rx_head = int(device_load(&q.rx_head.value));
                 const bool tx_backlog = tx_head < int(device_load(&q.tx_tail.value));
-                const bool rx_backlog = rx_head < int(device_load(&q.rx_tail.value));
+                bool rx_backlog = rx_head < int(device_load(&q.rx_tail.value));
+                // Receive tickets are there long before the first row may be requested (rx_row
+                // holds the gate).  Only the first kPreGateRows of them are claimed ahead of
+                // it, by wavefronts that then wait with their addresses ready: if every
+                // wavefront did, they would all fire at once and each would have its first
+                // row after the time the link needs for all of them, with nobody left to transmit.
+                // ... and until the transmit side has its first rows on their way: a row written
+                // behind a link full of requested rows is acknowledged after all of them, and a
+                // dispatch of a few rows would then end with that acknowledgement, the peers'
+                // answer and the drain instead of with its last received row.
+                if (rx_backlog && !gate_seen && rx_head >= kPreGateRows) {
+                    const int tx_known = device_load(&q.tx_head.total);
+                    gate_seen = (device_load(state.receive_prefix_state) & kPrefixRequested) &&
+                                (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch)) &&
+                                tx_known >= 0 && int(device_load(&q.tx_tail.value)) >= (tx_known < 4 * kMinTxWaves ? tx_known : 4 * kMinTxWaves);
+                    rx_backlog = gate_seen != 0;
+                }
                 const int tx_total = device_load(&q.tx_head.total), rx_total = device_load(&q.rx_head.total);
                 const bool tx_done = tx_total >= 0 && tx_head >= tx_total, rx_done = rx_total >= 0 && rx_head >= rx_total;
                 // Totals unknown: a handful of wavefronts start to transmit, the others
@@ -1305,10 +1318,14 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
             }
         }
         choice = broadcast_first(choice);
+        gate_open = broadcast_first(gate_seen) != 0;
         if (choice < 0) break;
         if (choice == 0) {
             PCIE_EP_PROFILE(if (!idle_begin) idle_begin = profile.now();)
-            backoff();
+            // Every look is seven loads of the queue counters; a couple of hundred idle wavefronts
+            // looking four times a microsecond would keep the producers' own updates of those
+            // counters waiting.  About a microsecond between looks.
+            __builtin_amdgcn_s_sleep(32);
             continue;
         }
         PCIE_EP_PROFILE(if (idle_begin) { profile.add(kProfileIdleSum, profile.now() - idle_begin); idle_begin = 0; })
@@ -1325,7 +1342,7 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
         PCIE_EP_PROFILE(profile.add(kProfileTicketWaitSum, profile.now() - claim_begin); const bool sampled = rows_moved++ % kProfileSampleStride == 0;
                         if (sampled) profile.add(transmit ? kProfileSampledTxRows : kProfileSampledRxRows); profile.add(transmit ? kProfileTxRows : kProfileRxRows);)
         const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters PCIE_EP_PROFILE(, profile, sampled))
-                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, prefixes_known PCIE_EP_PROFILE(, profile, sampled));
+                                    : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, deadline, gate_open, prefixes_known PCIE_EP_PROFILE(, profile, sampled));
         PCIE_EP_PROFILE(profile.last(kProfileLastRowNs);)
         if (!go_on) break;
     }
@@ -1362,7 +1379,8 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
     __shared__ WaveScratch lds;
     extern __shared__ __align__(16) unsigned char prologue_lds[];  // sized by the launcher when the prologue rides in this launch
     const int channels = state.z.dims.channels;
-    int block = blockIdx.x;
+    int block = transport_block(transport_grid(state), int(blockIdx.x));
+    if (block < 0) return;  // a filler id
     int wave = threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
     uint32_t* scratch = lds.words[wave];
@@ -1381,8 +1399,12 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
         // Workgroup 0 begins the epoch, the ones after it lay out one chunk of tokens each.
         if (block < prologue_groups) {
             if (block == 0) {
+                // The helpers' findings: zeroed before any wavefront of the workgroup goes its own way.
+                __shared__ int findings[kTransportMaxThreads / kWave];
+                if (threadIdx.x < kTransportMaxThreads / kWave) findings[threadIdx.x] = 0;
+                __syncthreads();
+                epoch_begin_role(state, wave, lane, waves_per_group, findings);
                 if (wave >= 2) return;
-                epoch_begin_role(state, wave, lane);
                 return finish_role(state, q, lane, roles);
             }
             prologue_chunk<8, true>(state, prologue_lds, waves_per_group, state.prologue_chunks, block - 1);
@@ -1394,21 +1416,41 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
     } else if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) {
         return;  // the prologue kernel in front of this one failed
     }
-    if (block >= channels + payload_groups) {
+    const int channel_groups = control_groups(state);
+    if (block >= channel_groups + payload_groups) {
         if (begun) local_rows<kVector>(state, q, lane);
         return finish_role(state, q, lane, roles);
     }
-    if (block < channels) {
+    if (block < channel_groups) {
+        if (payload_groups) {
+            // Control workgroups of their own: the two control XCDs alternate over their
+            // ids, and a workgroup holds the controls of ONE direction for a pair of
+            // channels (wavefront w: channel 2 * pair + w), transmit on one XCD, receive
+            // on the other.  A receive control polls descriptors in host memory all the
+            // time, and each of those reads stays in its XCD's memory queues for as long
+            // as the row reads in front of it on the link take; the transmit controls,
+            // the producer of the prefixes and the prologue only touch device memory
+            // while rows flow and must not wait behind them.
+            const bool transmit = (block + prologue_groups) % kControlXcds == 0;
+            const int pair = block / 2, channel = 2 * pair + wave;
+            if (wave < 2) {
+                if (channel >= channels) return;
+                if (begun) {
+                    if (transmit) tx_control(state, q, channel, lane);
+                    else rx_control(state, q, channel, lane);
+                }
+                return finish_role(state, q, lane, roles);
+            }
+            // The producer of the receive prefixes: third wavefront of the first transmit control workgroup.
+            if (pair != 0 || !transmit || wave != 2 || !dedicated_prefix_producer(state)) return;
+            if (begun) receive_prefix_role(state, lane);
+            return finish_role(state, q, lane, roles);
+        }
         if (wave < 2) {
             if (begun) {
                 if (wave == 0) tx_control(state, q, block, lane);
                 else rx_control(state, q, block, lane);
             }
-            return finish_role(state, q, lane, roles);
-        }
-        if (payload_groups) {
-            if (block != 0 || wave != 2 || !dedicated_prefix_producer(state)) return;
-            if (begun) receive_prefix_role(state, lane);
             return finish_role(state, q, lane, roles);
         }
         wave -= 2;
@@ -1417,7 +1459,7 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
     // Position of this wavefront among all payload wavefronts, wavefront-major: a
     // direction's share is spread over the workgroups before it doubles up in one.
     const int groups = payload_groups ? payload_groups : channels;
-    const int group = payload_groups ? block - channels : block;
+    const int group = payload_groups ? block - channel_groups : block;
     if (begun) payload_worker<kFp8, kVector>(state, q, scratch, lane, wave * groups + group, groups * payload_waves);
     finish_role(state, q, lane, roles);
     // Every role loop has an explicit completion, abort or timeout exit and no
@@ -1447,9 +1489,7 @@ hipError_t transport_workgroups_per_unit(const DeviceState& state, int* per_unit
 }
 
 hipError_t launch_transport(const DeviceState& state, hipStream_t stream) {
-    const int prologue_groups = fused_prologue_groups(state);
-    const dim3 grid(prologue_groups + state.z.dims.channels + (state.worker_groups > 0 ? state.worker_groups : 0) + state.local_groups),
-        block(transport_threads(state));
+    const dim3 grid(transport_grid(state).blocks), block(transport_threads(state));
     if (int(block.x) > kTransportMaxThreads) return hipErrorInvalidValue;
     size_t dynamic_lds = 0;
     if (state.fused) {

@@ -25,10 +25,10 @@ from . import _native
 
 COMMON = ("enter_ns", "exit_ns", "total_ns", "items")
 CONTROL = COMMON + ("first_ticket_ns", "last_ticket_ns", "workers_done_ns", "drained_ns", "finished_ns", "polls", "poll_misses",
-                    "poll_sum", "health_scans", "health_sum", "counts_known_ns", "gate_open_ns", "prefix_enter_ns",
+                    "poll_sum", "health_scans", "health_sum", "counts_known_ns", "spare", "prefix_enter_ns",
                     "prefix_counts_ready_ns", "prefix_mailbox_ns", "prefix_published_ns")
 WORKER = COMMON + ("first_claim_ns", "last_row_ns", "tx_rows", "rx_rows", "sampled_tx_rows", "sampled_rx_rows", "ticket_wait_sum",
-                   "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum")
+                   "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum", "gate_open_ns")
 PROLOGUE = COMMON + ("layout_ns", "totals_ns", "verdict_ns", "mailbox_free_ns", "mailbox_acked_ns", "counts_ready_ns",
                      "begun_ns", "routes_ns", "masks_ns", "chunk_totals_ns", "plan_ready_ns")
 
@@ -91,7 +91,7 @@ def timeline(records: Dict[str, np.ndarray]) -> Dict[str, float]:
         "transport.first_role_enter": first(np.concatenate([_col(txc, CONTROL, "enter_ns"), _col(rxc, CONTROL, "enter_ns"), _col(wrk, WORKER, "enter_ns")])),
         "prefix.enter": first(_col(rxc, CONTROL, "prefix_enter_ns")), "prefix.counts_ready_seen": first(_col(rxc, CONTROL, "prefix_counts_ready_ns")),
         "prefix.mailboxes_returned": first(_col(rxc, CONTROL, "prefix_mailbox_ns")), "prefix.published": first(_col(rxc, CONTROL, "prefix_published_ns")),
-        "rx.first_gate_open": first(_col(rxc, CONTROL, "gate_open_ns")), "rx.first_ticket": first(_col(rxc, CONTROL, "first_ticket_ns")),
+        "rx.first_gate_open": first(_col(wrk, WORKER, "gate_open_ns")), "rx.first_ticket": first(_col(rxc, CONTROL, "first_ticket_ns")),
         "rx.last_ticket": last(_col(rxc, CONTROL, "last_ticket_ns")), "rx.counts_known_first": first(_col(rxc, CONTROL, "counts_known_ns")),
         "rx.rows_scattered_last": last(_col(rxc, CONTROL, "workers_done_ns")), "rx.finished_last": last(_col(rxc, CONTROL, "finished_ns")),
         "rx.descriptor_poll_us": per(_col(rxc, CONTROL, "poll_sum"), _col(rxc, CONTROL, "polls")),
