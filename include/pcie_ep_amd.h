@@ -148,6 +148,33 @@ int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes);
  * `peer_threads > 0`, the host peer emulator. */
 int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** runtime);
 
+/* The pinned segments of a whole EP world as a set that several runtimes share:
+ * one segment per rank (pcie_ep_sizes.segment_bytes each) and, in relay mode, the
+ * replica payload regions [rank * 8 + domain] (pcie_ep_sizes.replica_region_bytes
+ * each).  Pointers are what the GPU uses (for pinned, mapped host memory the host
+ * address).  Replaces the set of /dev/shm segments a rank creates and its peers
+ * map (create_advanced_segments / AdvancedSharedMemory,
+ * csrc/comm/advanced_shared_memory.hpp:143-233). */
+typedef struct pcie_ep_segments {
+    void* segment[16];
+    void* replica[16 * 8];
+} pcie_ep_segments;
+
+/* Allocates (pinned, fine-grained, GPU-mapped, zeroed; NUMA placement as
+ * pcie_ep_runtime_create does it) and frees such a set in this process. */
+int pcie_ep_segments_create(const pcie_ep_config* config, pcie_ep_segments* segments);
+int pcie_ep_segments_destroy(pcie_ep_segments* segments);
+
+/* pcie_ep_runtime_create for rank `config->local_rank` on segments it does not
+ * own: every other rank of `segments` is a runtime of its own (another stream,
+ * another process that mapped the same memory, another GPU), so `peer_threads`
+ * must be 0 and no emulator is started.  The set must outlive the runtime and
+ * must have been zeroed before its first user.  Replaces the attach path of the
+ * reference's runtime (attach_advanced_segments / register_advanced_segments,
+ * csrc/comm/advanced_shared_memory.hpp:235-288; its use by the constructor,
+ * csrc/buffers/advanced.hpp:107-124). */
+int pcie_ep_runtime_attach(const pcie_ep_config* config, const pcie_ep_segments* segments, pcie_ep_runtime** runtime);
+
 /* Replaces AdvancedRuntime::close (advanced.hpp:229-240).  The caller must have
  * synchronised every stream that ran a dispatch. */
 int pcie_ep_runtime_destroy(pcie_ep_runtime* runtime);
@@ -271,6 +298,13 @@ int pcie_ep_dequantize_fp8(const uint8_t* codes, const float* scales, void* out,
  * the unique rows of `args` into its expert-major outputs using the prefixes
  * already present in `args` (what a non-fused dispatch launches last). */
 int pcie_ep_expand_unique(pcie_ep_runtime* runtime, const pcie_ep_dispatch_args* args, void* stream);
+
+/* Launches an instantiated HIP graph (a hipGraphExec_t, e.g. the one a captured
+ * dispatch was turned into) on `stream`.  For hosts whose graph object can only
+ * replay on "the current stream" of their framework: switching that stream around
+ * every replay costs more CPU time than a small dispatch takes on the GPU.
+ * No counterpart in the reference (its graph.py:150-202 replays through PyTorch). */
+int pcie_ep_graph_launch(void* graph_exec, void* stream);
 
 /* Per-kernel timing with HIP events recorded on the dispatch stream (off by
  * default; must stay off for a dispatch that is being captured into a graph).

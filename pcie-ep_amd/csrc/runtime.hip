@@ -246,6 +246,7 @@ struct pcie_ep_runtime {
     // Relay mode: replica payload regions [rank][domain], each bound to its
     // domain's node when that node exists here, and this rank's relay workers.
     char* replica[kMaxRanks * kMaxDomains] = {};
+    bool owns_segments = true;  // false: attached to segments of a pcie_ep_segments set, which outlives this runtime
     int domain_node[kMaxDomains] = {};
     bool domain_bound[kMaxDomains] = {};
     std::unique_ptr<NumaRelay> relay;
@@ -427,7 +428,86 @@ int pcie_ep_query_sizes(const pcie_ep_config* config, pcie_ep_sizes* sizes) {
     return 0;
 }
 
-int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) {
+namespace {
+
+// Allocates the pinned segments of every rank (and, in relay mode, the replica
+// regions): first touch by this thread under the requested NUMA policy, then
+// zeroed - a zero sequence word means "never written".  A rank's segment belongs
+// on the rank's own node and each replica payload region on the node of the
+// domain it serves (advanced_shared_memory.hpp:214-262); a node that this machine
+// does not have leaves the memory where first touch puts it.
+int allocate_segments(const pcie_ep_config& config, const Dimensions& dims, const SegmentLayout& z, char** segments, char** replica,
+                      int* domain_node, bool* domain_bound) {
+    int status = 0;
+    if (dims.domains) {
+        int rank_domain[kMaxRanks];
+        numa_domains(config, domain_node, rank_domain);
+    }
+    for (int rank = 0; rank < dims.num_ranks && !status; ++rank) {
+        int node = config.staging_numa_node;
+        if (node < 0 && dims.domains && numa_node_exists(config.rank_numa_nodes[rank])) node = config.rank_numa_nodes[rank];
+        status = pinned_zeroed(z.size_bytes, node, &segments[rank], "source segment");
+        for (int domain = 0; domain < dims.domains && !status; ++domain) {
+            const bool present = numa_node_exists(domain_node[domain]);
+            domain_bound[domain] = present;
+            status = pinned_zeroed(z.replica_region_bytes, present ? domain_node[domain] : -1, &replica[rank * kMaxDomains + domain], "replica region");
+        }
+    }
+    return status;
+}
+
+int free_segments(char** segments, char** replica) {
+    int status = 0;
+    for (int rank = 0; rank < kMaxRanks; ++rank) {
+        if (segments[rank] && hipHostFree(segments[rank]) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a source segment failed");
+        segments[rank] = nullptr;
+    }
+    for (int index = 0; index < kMaxRanks * kMaxDomains; ++index) {
+        if (replica[index] && hipHostFree(replica[index]) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a replica region failed");
+        replica[index] = nullptr;
+    }
+    return status;
+}
+
+int create_runtime(const pcie_ep_config* config, const pcie_ep_segments* attached, pcie_ep_runtime** out);
+
+}  // namespace
+
+int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) { return create_runtime(config, nullptr, out); }
+
+int pcie_ep_runtime_attach(const pcie_ep_config* config, const pcie_ep_segments* segments, pcie_ep_runtime** out) {
+    if (!segments) return set_error(PCIE_EP_E_INVALID, "segments is NULL");
+    return create_runtime(config, segments, out);
+}
+
+int pcie_ep_segments_create(const pcie_ep_config* config, pcie_ep_segments* out) {
+    Dimensions dims;
+    if (int status = check_config(config, dims)) return status;
+    if (!out) return set_error(PCIE_EP_E_INVALID, "segments output pointer is NULL");
+    int device_count = 0;
+    if (hipGetDeviceCount(&device_count) != hipSuccess || device_count <= config->device)
+        return set_error(PCIE_EP_E_HIP, "no HIP device %d is available: the host-staged runtime needs a GPU", config->device);
+    HIP_TRY(hipSetDevice(config->device));
+    std::memset(out, 0, sizeof *out);
+    static_assert(sizeof(out->segment) / sizeof(void*) == kMaxRanks && sizeof(out->replica) / sizeof(void*) == kMaxRanks * kMaxDomains,
+                  "pcie_ep_segments is sized by the wire limits");
+    const SegmentLayout z = make_segment_layout(dims);
+    int domain_node[kMaxDomains] = {};
+    bool domain_bound[kMaxDomains] = {};
+    const int status = allocate_segments(*config, dims, z, reinterpret_cast<char**>(out->segment), reinterpret_cast<char**>(out->replica), domain_node,
+                                         domain_bound);
+    if (status) (void)free_segments(reinterpret_cast<char**>(out->segment), reinterpret_cast<char**>(out->replica));
+    return status;
+}
+
+int pcie_ep_segments_destroy(pcie_ep_segments* segments) {
+    if (!segments) return 0;
+    return free_segments(reinterpret_cast<char**>(segments->segment), reinterpret_cast<char**>(segments->replica));
+}
+
+namespace {
+
+int create_runtime(const pcie_ep_config* config, const pcie_ep_segments* attached, pcie_ep_runtime** out) {
     Dimensions dims;
     if (int status = check_config(config, dims)) return status;
     if (!out) return set_error(PCIE_EP_E_INVALID, "runtime output pointer is NULL");
@@ -466,27 +546,29 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     }
 
     // Pinned, fine-grained, GPU-mapped segments (the reference registers
-    // /dev/shm mappings: advanced_shared_memory.hpp:264-288).  First touch is
-    // by this thread under the requested NUMA policy, then zeroed: a zero
-    // sequence word means "never written".  In relay mode a rank's segment
-    // belongs on the rank's own node and each replica payload region on the node
-    // of the domain it serves (advanced_shared_memory.hpp:214-262); a node that
-    // this machine does not have leaves the memory where first touch puts it.
+    // /dev/shm mappings: advanced_shared_memory.hpp:264-288): this runtime's own, or
+    // those of a set that several runtimes share (advanced_shared_memory.hpp:235-262:
+    // attach validates the header a creator wrote; here the creator's struct is the
+    // proof, and what is checked is that every pointer this rank will use is there).
     int status = 0;
-    if (dims.domains) {
-        int rank_domain[kMaxRanks];
-        numa_domains(*config, rt->domain_node, rank_domain);
-    }
-    for (int rank = 0; rank < dims.num_ranks && !status; ++rank) {
-        int node = config->staging_numa_node;
-        if (node < 0 && dims.domains && numa_node_exists(config->rank_numa_nodes[rank])) node = config->rank_numa_nodes[rank];
-        status = pinned_zeroed(rt->z.size_bytes, node, &rt->segments[rank], "source segment");
-        for (int domain = 0; domain < dims.domains && !status; ++domain) {
-            const bool present = numa_node_exists(rt->domain_node[domain]);
-            rt->domain_bound[domain] = present;
-            status = pinned_zeroed(rt->z.replica_region_bytes, present ? rt->domain_node[domain] : -1, &rt->replica[rank * kMaxDomains + domain],
-                                   "replica region");
+    if (attached) {
+        if (config->peer_threads > 0)
+            return set_error(PCIE_EP_E_INVALID, "an attached runtime has real peers: peer_threads must be 0");
+        rt->owns_segments = false;
+        if (dims.domains) {
+            int rank_domain[kMaxRanks];
+            numa_domains(*config, rt->domain_node, rank_domain);
         }
+        for (int rank = 0; rank < dims.num_ranks; ++rank) {
+            rt->segments[rank] = static_cast<char*>(attached->segment[rank]);
+            if (!rt->segments[rank]) return set_error(PCIE_EP_E_INVALID, "segment of rank %d is NULL", rank);
+            for (int domain = 0; domain < dims.domains; ++domain) {
+                rt->replica[rank * kMaxDomains + domain] = static_cast<char*>(attached->replica[rank * kMaxDomains + domain]);
+                if (!rt->replica[rank * kMaxDomains + domain]) return set_error(PCIE_EP_E_INVALID, "replica region %d of rank %d is NULL", domain, rank);
+            }
+        }
+    } else {
+        status = allocate_segments(*config, dims, rt->z, rt->segments, rt->replica, rt->domain_node, rt->domain_bound);
     }
     if (!status) {
         const size_t history = size_t(dims.channels) * ((dims.max_tokens + dims.channels - 1) / dims.channels) * 4;
@@ -509,10 +591,7 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
         if (error != hipSuccess) status = set_error(PCIE_EP_E_HIP, "device workspace allocation failed: %s", hipGetErrorString(error));
     }
     if (status) {
-        for (char* segment : rt->segments)
-            if (segment) (void)hipHostFree(segment);
-        for (char* region : rt->replica)
-            if (region) (void)hipHostFree(region);
+        if (rt->owns_segments) (void)free_segments(rt->segments, rt->replica);
         if (rt->epoch) (void)hipFree(rt->epoch);
         if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
         if (rt->queues) (void)hipFree(rt->queues);
@@ -538,6 +617,8 @@ int pcie_ep_runtime_create(const pcie_ep_config* config, pcie_ep_runtime** out) 
     return 0;
 }
 
+}  // namespace
+
 int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     if (!rt) return 0;
     rt->closed = true;
@@ -547,14 +628,7 @@ int pcie_ep_runtime_destroy(pcie_ep_runtime* rt) {
     rt->peers.reset();  // joins the emulator threads before the segments go away
     rt->relay.reset();
     int status = 0;
-    for (char*& segment : rt->segments) {
-        if (segment && hipHostFree(segment) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a source segment failed");
-        segment = nullptr;
-    }
-    for (char*& region : rt->replica) {
-        if (region && hipHostFree(region) != hipSuccess) status = set_error(PCIE_EP_E_HIP, "hipHostFree of a replica region failed");
-        region = nullptr;
-    }
+    if (rt->owns_segments) status = free_segments(rt->segments, rt->replica);
     if (rt->epoch) (void)hipFree(rt->epoch);
     if (rt->chan_remote_tokens) (void)hipFree(rt->chan_remote_tokens);
     if (rt->queues) (void)hipFree(rt->queues);
@@ -689,6 +763,12 @@ int pcie_ep_profile_read(pcie_ep_runtime* rt, int64_t* records) {
     if (!records) return set_error(PCIE_EP_E_INVALID, "bad profile arguments");
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(records, rt->profiling, size_t(rt->profile_row_count) * kProfileFields * sizeof(int64_t), hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int pcie_ep_graph_launch(void* graph_exec, void* stream) {
+    if (!graph_exec) return set_error(PCIE_EP_E_INVALID, "graph_exec is NULL");
+    HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), static_cast<hipStream_t>(stream)));
     return 0;
 }
 

@@ -1250,7 +1250,7 @@ constexpr int64_t kTxWeight = 9, kRxWeight = 4;
 constexpr int64_t kTxLeadBytes = 24 << 20;
 constexpr int kMinTxWaves = 16;
 constexpr uint64_t kIdleCrossoverUs = 30;
-constexpr int kPreGateRows = 16;
+constexpr int kPreGateRows = 32;
 
 template <bool kFp8, bool kVector>
 __device__ __forceinline__ void payload_worker(const DeviceState& state, TransportQueues& q, uint32_t* scratch, int lane, int order, int waves) {
@@ -1276,22 +1276,16 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
                 // it, by wavefronts that then wait with their addresses ready: if every
                 // wavefront did, they would all fire at once and each would have its first
                 // row after the time the link needs for all of them, with nobody left to transmit.
-                // ... and until the transmit side has its first rows on their way: a row written
-                // behind a link full of requested rows is acknowledged after all of them, and a
-                // dispatch of a few rows would then end with that acknowledgement, the peers'
-                // answer and the drain instead of with its last received row.
                 if (rx_backlog && !gate_seen && rx_head >= kPreGateRows) {
-                    const int tx_known = device_load(&q.tx_head.total);
                     gate_seen = (device_load(state.receive_prefix_state) & kPrefixRequested) &&
-                                (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch)) &&
-                                tx_known >= 0 && int(device_load(&q.tx_tail.value)) >= (tx_known < 4 * kMinTxWaves ? tx_known : 4 * kMinTxWaves);
+                                (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch));
                     rx_backlog = gate_seen != 0;
                 }
                 const int tx_total = device_load(&q.tx_head.total), rx_total = device_load(&q.rx_head.total);
                 const bool tx_done = tx_total >= 0 && tx_head >= tx_total, rx_done = rx_total >= 0 && rx_head >= rx_total;
                 // Totals unknown: a handful of wavefronts start to transmit, the others
                 // wait for the first descriptors.
-                bool prefer_tx = order < kMinTxWaves;
+                bool prefer_tx = order < kMinTxWaves && 2 * order < waves;
                 if (tx_total >= 0 && rx_total >= 0) {
                     const int rx_rows = rx_total - rx_head - (lead < rx_total / 4 ? lead : rx_total / 4);
                     const int64_t tx_left = tx_done ? 0 : kTxWeight * (tx_total - tx_head), rx_left = rx_rows > 0 ? kRxWeight * rx_rows : 0;
@@ -1304,7 +1298,13 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
                 else if (other_backlog) {
                     const uint64_t now = now_ticks();
                     if (!idle_since) idle_since = now;
-                    if (own_done || now - idle_since > kIdleCrossoverUs * state.clock_khz / 1000) choice = prefer_tx ? 2 : 1;
+                    // Towards the receive side after a while; towards the transmit side only once
+                    // everything has been received.  A transmit row waits for its receivers (slot ACK,
+                    // descriptor credit); if every wavefront of a rank could end up in such a wait, two
+                    // ranks whose receivers are each other's kernels could wait for each other for ever.
+                    // The wavefronts that do not transmit by the rule above (at least half of them)
+                    // therefore never do while a row may still come in.
+                    if (own_done || (prefer_tx && now - idle_since > kIdleCrossoverUs * state.clock_khz / 1000)) choice = prefer_tx ? 2 : 1;
                 }
                 if (choice) idle_since = 0;
                 else {

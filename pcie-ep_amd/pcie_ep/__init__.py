@@ -9,6 +9,7 @@ from .config import HostStagedConfig
 from .graph import GraphDispatch
 from .handle import CachedLayout, EPHandle, HostStagedEPHandle
 from .overlap import EventOverlap
+from .runtime import SharedSegments
 
 __all__ = [
     "EPBuffer",
@@ -20,6 +21,7 @@ __all__ = [
     "topk_idx_t",
     "GraphDispatch",
     "CachedLayout",
+    "SharedSegments",  # this build: the ranks of one process share one set of host segments
 ]
 
 topk_idx_t = torch.int64

@@ -29,6 +29,10 @@ class Config(C.Structure):
         ("reserved", C.c_int32 * 4), ("rank_numa_nodes", C.c_int32 * 16), ("relay_cpus", C.c_int32 * 64), ("relay_delay_ns", C.c_uint64)]
 
 
+class Segments(C.Structure):
+    _fields_ = [("segment", C.c_void_p * 16), ("replica", C.c_void_p * 128)]
+
+
 class Sizes(C.Structure):
     _fields_ = [
         ("unique_rows", C.c_int64), ("expanded_rows", C.c_int64), ("plan_bytes", C.c_int64), ("segment_bytes", C.c_int64),
@@ -101,6 +105,10 @@ _PROTOTYPES = {
     "pcie_ep_dequantize_fp8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "pcie_ep_profile_shape": (C.c_int, [C.c_void_p] + [C.POINTER(C.c_int32)] * 4),
     "pcie_ep_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "pcie_ep_graph_launch": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "pcie_ep_segments_create": (C.c_int, [C.POINTER(Config), C.POINTER(Segments)]),
+    "pcie_ep_segments_destroy": (C.c_int, [C.POINTER(Segments)]),
+    "pcie_ep_runtime_attach": (C.c_int, [C.POINTER(Config), C.POINTER(Segments), C.POINTER(C.c_void_p)]),
     "pcie_ep_set_kernel_timing": (C.c_int, [C.c_void_p, C.c_int32]),
     "pcie_ep_get_kernel_times": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "pcie_ep_measure_pinned_copy": (C.c_int, [C.c_int32, C.c_int64, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -46,11 +46,12 @@ _next_buffer_id = itertools.count(1)
 class _Ordering:
     """Stream ordering of one buffer."""
 
-    def __init__(self, device: int, compute_units: int = 0) -> None:
+    def __init__(self, device: int, compute_units: int = 0, stream: Any = None) -> None:
         self.device = device
-        # Optionally confine the dispatch kernels to the first `compute_units` units.
-        self.masked = MaskedStream(device, compute_units) if compute_units else None
-        self.stream = self.masked.stream if self.masked else torch.cuda.Stream(device=device)
+        # Optionally confine the dispatch kernels to the first `compute_units` units,
+        # or run them on a stream the caller brings.
+        self.masked = MaskedStream(device, compute_units) if compute_units and stream is None else None
+        self.stream = stream if stream is not None else (self.masked.stream if self.masked else torch.cuda.Stream(device=device))
         self.stream.wait_stream(torch.cuda.current_stream(device))
         self._stream_key = self._key(self.stream)
         self.raw_stream = int(self.stream.cuda_stream)
@@ -143,7 +144,9 @@ class HostStagedEPBuffer:
         worker_groups: int = 0,
         rank_numa_nodes: Optional[Tuple[int, ...]] = None,
         comm_stream_cus: int = 0,
+        comm_stream: Any = None,
         split_launch: bool = False,
+        shared_segments: Any = None,
     ) -> None:
         """Allocate the pinned host rings, the result pools and the peer emulator.
 
@@ -175,6 +178,20 @@ class HostStagedEPBuffer:
         default it rides in the transport kernel's launch wherever it fits (top-k up
         to 8, default launch shape), so that a dispatch is one launch and the receive
         side starts while the layout is computed.
+        ``comm_stream`` makes a stream of the caller's the communication stream (for
+        instance ``pcie_ep.streams.masked_stream(count, first).stream``: a stream on a
+        range of compute units, which has a hardware queue of its own, whereas
+        ordinary streams may be put behind one another on one queue).
+        ``shared_segments`` (a ``pcie_ep.SharedSegments``) attaches this rank to host
+        segments that the buffers of the other ranks use as well, instead of
+        allocating its own with emulated peers (the reference's ranks map each
+        other's ``/dev/shm`` segments: csrc/comm/advanced_shared_memory.hpp:235-288);
+        no peer emulator is started.  All ranks must then dispatch: a rank's
+        dispatch completes only when its peers have run theirs.  Ranks that share a
+        GPU must have their dispatches in flight together: each needs a communication
+        stream with a hardware queue of its own (``comm_stream``), and nothing that
+        synchronises with those streams (a synchronous copy, work on the legacy
+        default stream, which waits for masked streams) may be submitted between them.
         """
         if not torch.cuda.is_available():
             raise RuntimeError("Host-staged EP requires a ROCm GPU")
@@ -211,9 +228,15 @@ class HostStagedEPBuffer:
         self._state = "live"  # "live" -> "failed" | "closed"
         self._last_handle: Optional[HostStagedEPHandle] = None
         self._graph_capture = None
-        self._ordering = _Ordering(self.device, comm_stream_cus)
+        if comm_stream is not None and comm_stream_cus:
+            raise ValueError("comm_stream and comm_stream_cus exclude each other")
+        self._ordering = _Ordering(self.device, comm_stream_cus, comm_stream)
         self.runtime: Optional[NativeRuntime] = None
         threads = min(num_ranks - 1, 7) if peer_threads is None else peer_threads
+        if shared_segments is not None:
+            if peer_threads:
+                raise ValueError("a buffer on shared segments has real peers: peer_threads must be 0")
+            threads = 0
         if rank_numa_nodes is not None:
             if self.config.numa_mode != "relay":
                 raise ValueError("rank_numa_nodes is meaningful only with numa_mode='relay'")
@@ -222,7 +245,7 @@ class HostStagedEPBuffer:
         self.runtime = NativeRuntime(rank, num_ranks, num_max_tokens_per_rank, hidden, num_topk, num_experts, self.config,
                                      self.device, peer_threads=threads, staging_numa_node=staging_numa_node,
                                      tx_waves=tx_waves, rx_waves=rx_waves, worker_groups=worker_groups,
-                                     rank_numa_nodes=rank_numa_nodes, split_launch=split_launch)
+                                     rank_numa_nodes=rank_numa_nodes, split_launch=split_launch, shared_segments=shared_segments)
         if comm_stream_cus:
             # Control and payload workgroups wait for each other through device memory:
             # the masked units must hold all of them at once, or every dispatch would

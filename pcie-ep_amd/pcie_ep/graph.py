@@ -17,10 +17,12 @@ ordering, consumer tracking and result wrapping exist once.
 
 from __future__ import annotations
 
+import ctypes as C
 from typing import Any, Dict, Optional
 
 import torch
 
+from . import _native
 from .handle import memory_signature
 from .overlap import record_tensors
 from .request import DispatchRequest, admit
@@ -32,6 +34,13 @@ class GraphDispatch:
         self._generation = owner._generation
         self._frozen = tuple(memory_signature(t) if t is not None else None for t in request.inputs)
         self._open = True
+        # The instantiated graph is launched on the communication stream directly
+        # (torch's own replay launches on the current stream, and making the
+        # communication stream current around every replay is a measurable part of
+        # a small replay's CPU time).
+        self._exec = C.c_void_p(int(graph.raw_cuda_graph_exec()))
+        self._launch_exec = _native.library().pcie_ep_graph_launch
+        self._raw_stream = C.c_void_p(int(owner.get_comm_stream().cuda_stream))
 
     # The captured inputs under the reference's attribute names.
     x = property(lambda self: self._request.x)
@@ -58,10 +67,10 @@ class GraphDispatch:
                 raise RuntimeError("GraphDispatch.replay cannot be nested in another capture")
 
             def replayed() -> Dict[str, Any]:
-                self._graph.replay()
+                _native.check(self._launch_exec(self._exec, self._raw_stream), invalid=RuntimeError)
                 return self._result
 
-            return owner._launch(self._request, replayed, (self,), previous_event, async_with_compute_stream)
+            return owner._launch(self._request, replayed, (self,), previous_event, async_with_compute_stream, through_torch=False)
 
     def close(self) -> None:
         if self._open:

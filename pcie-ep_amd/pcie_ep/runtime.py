@@ -39,6 +39,44 @@ class RoutePlan:
         self.storage = torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
+class SharedSegments:
+    """The pinned host segments of a whole EP world, shared by the runtimes of its
+    ranks (the set of ``/dev/shm`` segments of the reference, which every rank maps:
+    csrc/comm/advanced_shared_memory.hpp:143-288).  The first buffer constructed
+    with an empty set allocates it for its own dimensions; every further buffer
+    attaches and must have the same dimensions.  No host thread stands in for any
+    rank: every rank is a buffer of its own (here: on another stream of the GPU).
+    Close it after the buffers."""
+
+    def __init__(self) -> None:
+        self._native = None
+        self._signature = None
+        self._users = 0
+
+    def attach(self, lib, native_config, sizes) -> "C._Pointer":
+        signature = (native_config.num_ranks, int(sizes.segment_bytes), int(sizes.replica_region_bytes), int(sizes.num_domains),
+                     native_config.channels, native_config.payload_slots, native_config.descriptor_slots, native_config.max_tokens,
+                     native_config.hidden, native_config.topk, native_config.num_experts, native_config.wire_fp8)
+        if self._native is None:
+            self._native = _native.Segments()
+            _native.check(lib.pcie_ep_segments_create(C.byref(native_config), C.byref(self._native)), invalid=RuntimeError)
+            self._signature = signature
+        elif signature != self._signature:
+            raise ValueError("every buffer of a shared segment set must have the same dimensions and ring sizes")
+        self._users += 1
+        return C.byref(self._native)
+
+    def detach(self) -> None:
+        self._users -= 1
+
+    def close(self) -> None:
+        if self._native is not None:
+            if self._users > 0:
+                raise RuntimeError("close the buffers of a shared segment set before the set")
+            _native.check(_native.library().pcie_ep_segments_destroy(C.byref(self._native)), invalid=RuntimeError)
+            self._native = None
+
+
 class _Pool:
     """One preallocated set of result tensors.
 
@@ -73,8 +111,10 @@ class NativeRuntime:
 
     def __init__(self, rank: int, world: int, max_tokens: int, hidden: int, topk: int, experts: int, config: HostStagedConfig,
                  device: int, peer_threads: int = 0, staging_numa_node: int = -1, tx_waves: int = 0, rx_waves: int = 0,
-                 worker_groups: int = 0, rank_numa_nodes: Optional[tuple] = None, split_launch: bool = False) -> None:
+                 worker_groups: int = 0, rank_numa_nodes: Optional[tuple] = None, split_launch: bool = False,
+                 shared_segments: Optional[SharedSegments] = None) -> None:
         self._lib = _native.library()
+        self._shared_segments = None
         self.config = config
         self.device = torch.device("cuda", device)
         self.owner_id = next(_owner_ids)
@@ -104,7 +144,17 @@ class NativeRuntime:
         self.sizes = _native.Sizes()
         _native.check(self._lib.pcie_ep_query_sizes(C.byref(native), C.byref(self.sizes)), invalid=RuntimeError)
         handle = C.c_void_p()
-        _native.check(self._lib.pcie_ep_runtime_create(C.byref(native), C.byref(handle)), invalid=RuntimeError)
+        if shared_segments is None:
+            _native.check(self._lib.pcie_ep_runtime_create(C.byref(native), C.byref(handle)), invalid=RuntimeError)
+        else:
+            segments = shared_segments.attach(self._lib, native, self.sizes)
+            self._shared_segments = shared_segments
+            try:
+                _native.check(self._lib.pcie_ep_runtime_attach(C.byref(native), segments, C.byref(handle)), invalid=RuntimeError)
+            except Exception:
+                shared_segments.detach()
+                self._shared_segments = None
+                raise
         self._handle: Optional[C.c_void_p] = handle
         self.world, self.rank, self.hidden, self.topk = world, rank, hidden, topk
         self.max_tokens, self.experts = max_tokens, experts
@@ -343,4 +393,9 @@ class NativeRuntime:
         if self._handle is None:
             return
         handle, self._handle = self._handle, None
-        _native.check(self._lib.pcie_ep_runtime_destroy(handle), invalid=RuntimeError)
+        try:
+            _native.check(self._lib.pcie_ep_runtime_destroy(handle), invalid=RuntimeError)
+        finally:
+            if self._shared_segments is not None:
+                self._shared_segments.detach()
+                self._shared_segments = None
