@@ -364,9 +364,14 @@ int pcie_ep_measure_row_scatter(int32_t device, int32_t rows, int32_t row_bytes,
  * READY and ACK words 128 bytes apart, sequences from 1, a delayed last thread)
  * between this GPU and the calling CPU thread.  mode 0: one wavefront produces,
  * the CPU consumes; 1: a workgroup of four wavefronts produces; 2: the CPU
- * produces, one wavefront consumes; 3: a workgroup consumes.  Every round the
- * consumer compares every word of the payload with what the round must hold.
- * Mode 0 or 1 with PCIE_EP_LITMUS_PUBLISH_EARLY added is the negative control:
+ * produces, one wavefront consumes; 3: a workgroup consumes; 4: one wavefront
+ * produces and a wavefront of another kernel, on another stream, consumes (both
+ * ends on the GPU, the slot in host memory between them: the hand-off between
+ * two GPUs of a deployment, which is what the reference's program runs); 5: the
+ * same between two workgroups.  In modes 4 and 5 the gpu_* fields are the
+ * consumer kernel's verdict and the host_* fields the producer kernel's.  Every
+ * round the consumer compares every word of the payload with what the round must
+ * hold.  Mode 0, 1, 4 or 5 with PCIE_EP_LITMUS_PUBLISH_EARLY added is the negative control:
  * the producer publishes READY without waiting for its payload stores; with
  * other traffic on the host link the consumer then finds stale words (code 4),
  * which shows that the experiment can fail and that the wait is needed.

@@ -20,12 +20,20 @@
 //           (publish_counts -> peer)
 //   mode 2  the CPU produces, a wavefront consumes    (peer -> RX worker)
 //   mode 3  the CPU produces, a workgroup consumes
-//   mode 0 or 1 with flag 16: negative control - the producer publishes the
+//   mode 4  a wavefront produces, a wavefront of ANOTHER kernel on another stream
+//           consumes                                  (TX worker -> RX worker of a peer
+//           GPU: the hand-off a deployment performs, and the reference's experiment
+//           proper - both ends are kernels, the slot lies in host memory between them)
+//   mode 5  a workgroup produces, a workgroup of another kernel consumes
+//   mode 0, 1, 4 or 5 with flag 16: negative control - the producer publishes the
 //           sequence word WITHOUT waiting for its payload stores.  On an idle link
 //           posted writes of one compute unit arrive in order and nothing shows; with
 //           other traffic on the link the CPU finds words of an earlier round within
 //           thousands of rounds.  It shows that the experiment can fail, and that
 //           the wait it drops is needed, not merely sufficient.
+// The two kernels of modes 4 and 5 run on two streams with disjoint compute-unit
+// masks, which have hardware queues of their own (two ordinary streams may be put
+// on one queue, one kernel behind the other, and the first would wait in vain).
 // One slot, strict alternation: the producer waits for ACK == sequence before
 // it overwrites the payload.  Every wait is bounded; a side that fails raises
 // the abort word the other side polls, so the kernel always ends.
@@ -212,7 +220,8 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
     };
     const bool publish_early = (mode & 16) != 0;
     mode &= ~16;
-    if (!out || mode < 0 || mode > 3 || (publish_early && mode > 1) || iterations < 1 || payload_bytes < 16 || payload_bytes % 16 || payload_bytes > (1 << 24) ||
+    const bool both_kernels = mode == 4 || mode == 5;
+    if (!out || mode < 0 || mode > 5 || (publish_early && (mode == 2 || mode == 3)) || iterations < 1 || payload_bytes < 16 || payload_bytes % 16 || payload_bytes > (1 << 24) ||
         writer_delay_ns < 0 || reader_delay_ns < 0 || timeout_ms < 1)
         return fail(PCIE_EP_E_INVALID, "bad litmus arguments");
     std::memset(out, 0, sizeof *out);
@@ -224,12 +233,25 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
     const size_t bytes = 4 * 128 + size_t(payload_bytes);
     char* host = nullptr;
     int64_t* result = nullptr;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr, consumer_stream = nullptr;
     hipError_t status = hipHostMalloc(reinterpret_cast<void**>(&host), bytes, hipHostMallocCoherent | hipHostMallocMapped | hipHostMallocPortable);
     if (status == hipSuccess) std::memset(host, 0, bytes);
-    if (status == hipSuccess) status = hipMalloc(reinterpret_cast<void**>(&result), 3 * sizeof(int64_t));
-    if (status == hipSuccess) status = hipMemset(result, 0, 3 * sizeof(int64_t));
-    if (status == hipSuccess) status = hipStreamCreate(&stream);
+    // Two result records: [0..2] the kernel that the calling thread talks to (or the
+    // consumer kernel), [3..5] the producer kernel of the kernel-to-kernel modes.
+    if (status == hipSuccess) status = hipMalloc(reinterpret_cast<void**>(&result), 6 * sizeof(int64_t));
+    if (status == hipSuccess) status = hipMemset(result, 0, 6 * sizeof(int64_t));
+    if (status == hipSuccess && !both_kernels) status = hipStreamCreate(&stream);
+    if (status == hipSuccess && both_kernels) {
+        // Producer on the first half of the compute units, consumer on the second.
+        int units = 0;
+        status = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+        if (status == hipSuccess && units < 2) return fail(PCIE_EP_E_INVALID, "the kernel-to-kernel litmus needs two compute units");
+        uint32_t first[32] = {}, second[32] = {};
+        const int words = (units + 31) / 32 < 32 ? (units + 31) / 32 : 32;
+        for (int unit = 0; unit < units && unit < 1024; ++unit) (unit < units / 2 ? first : second)[unit / 32] |= 1u << (unit % 32);
+        if (status == hipSuccess) status = hipExtStreamCreateWithCUMask(&stream, uint32_t(words), first);
+        if (status == hipSuccess) status = hipExtStreamCreateWithCUMask(&consumer_stream, uint32_t(words), second);
+    }
     int64_t host_result[3] = {0, 0, -1};
     double elapsed = 0.0;
     if (status == hipSuccess) {
@@ -244,10 +266,18 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
         shared.writer_delay_ticks = uint64_t(writer_delay_ns) * uint64_t(clock_khz) / 1000000ull;
         shared.reader_delay_ticks = uint64_t(reader_delay_ns) * uint64_t(clock_khz) / 1000000ull;
         shared.timeout_ticks = uint64_t(timeout_ms) * uint64_t(clock_khz);
-        const bool gpu_produces = mode < 2, workgroup = (mode & 1) != 0;
+        const bool gpu_produces = mode < 2 || both_kernels, workgroup = (mode & 1) != 0;
         const dim3 grid(1), block(workgroup ? kRowKernelThreads : kWave);
         const auto start = Clock::now();
-        if (gpu_produces) {
+        if (both_kernels) {
+            // The consumer first: it only waits; then the producer, with a result record of its own.
+            if (workgroup) hipLaunchKernelGGL(litmus_consumer_kernel<true>, grid, block, 0, consumer_stream, shared);
+            else hipLaunchKernelGGL(litmus_consumer_kernel<false>, grid, block, 0, consumer_stream, shared);
+            status = hipGetLastError();
+            shared.result = result + 3;
+        }
+        if (status != hipSuccess) {
+        } else if (gpu_produces) {
             if (workgroup && publish_early) hipLaunchKernelGGL((litmus_producer_kernel<true, true>), grid, block, 0, stream, shared);
             else if (workgroup) hipLaunchKernelGGL((litmus_producer_kernel<true, false>), grid, block, 0, stream, shared);
             else if (publish_early) hipLaunchKernelGGL((litmus_producer_kernel<false, true>), grid, block, 0, stream, shared);
@@ -256,8 +286,13 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
             if (workgroup) hipLaunchKernelGGL(litmus_consumer_kernel<true>, grid, block, 0, stream, shared);
             else hipLaunchKernelGGL(litmus_consumer_kernel<false>, grid, block, 0, stream, shared);
         }
-        status = hipGetLastError();
-        if (status == hipSuccess) {
+        if (status == hipSuccess) status = hipGetLastError();
+        if (status == hipSuccess && both_kernels) {
+            status = hipStreamSynchronize(stream);
+            const hipError_t other = hipStreamSynchronize(consumer_stream);
+            if (status == hipSuccess) status = other;
+            elapsed = std::chrono::duration<double>(Clock::now() - start).count();
+        } else if (status == hipSuccess) {
             HostSide side{shared.payload, std::atomic_ref<uint64_t>(*shared.ready), std::atomic_ref<uint64_t>(*shared.ack),
                           std::atomic_ref<uint64_t>(*shared.abort_word), shared.vectors, timeout_ms};
             auto* words = reinterpret_cast<volatile uint32_t*>(shared.payload);
@@ -299,8 +334,14 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
             status = hipStreamSynchronize(stream);
             elapsed = std::chrono::duration<double>(Clock::now() - start).count();
         }
-        int64_t device_result[3] = {0, 0, -1};
+        int64_t device_result[6] = {0, 0, -1, 0, 0, -1};
         if (status == hipSuccess) status = hipMemcpy(device_result, result, sizeof device_result, hipMemcpyDeviceToHost);
+        if (both_kernels) {
+            // The producer kernel's verdict takes the place of the CPU side's.
+            host_result[0] = device_result[3];
+            host_result[1] = device_result[4];
+            host_result[2] = device_result[3] ? device_result[5] : -1;
+        }
         out->gpu_code = int32_t(device_result[0]);
         out->gpu_iteration = device_result[1];
         out->gpu_index = device_result[0] ? device_result[2] : -1;
@@ -311,6 +352,7 @@ int run_litmus(int device, int mode, int64_t iterations, int payload_bytes, int 
         out->seconds = elapsed;
     }
     if (stream) (void)hipStreamDestroy(stream);
+    if (consumer_stream) (void)hipStreamDestroy(consumer_stream);
     if (result) (void)hipFree(result);
     if (host) (void)hipHostFree(host);
     if (status != hipSuccess) return fail(PCIE_EP_E_HIP, hipGetErrorString(status));

@@ -2,8 +2,9 @@
 
 The reference ships a stand-alone two-GPU program for this
 (tests/mapped_litmus.cu, tests/MAPPED_LITMUS.md); here the same experiment runs
-between the GPU and the calling CPU thread, with the GPU side using the access
-primitives of the transport kernel.
+between the GPU and the calling CPU thread and between two kernels on two streams
+of the one GPU, with the GPU sides using the access primitives of the transport
+kernel.
 """
 
 from __future__ import annotations
@@ -18,6 +19,9 @@ from . import _native
 #: one wavefront produces, the CPU consumes / a workgroup produces / the CPU
 #: produces and one wavefront consumes / the CPU produces and a workgroup consumes
 GPU_WAVE_TO_CPU, GPU_GROUP_TO_CPU, CPU_TO_GPU_WAVE, CPU_TO_GPU_GROUP = 0, 1, 2, 3
+#: a wavefront (workgroup) of one kernel produces, a wavefront (workgroup) of another kernel on another stream consumes;
+#: the result's "gpu" entry is then the consumer kernel's verdict and "host" the producer kernel's
+GPU_WAVE_TO_GPU_WAVE, GPU_GROUP_TO_GPU_GROUP = 4, 5
 #: added to a GPU-produces mode: publish READY without waiting for the payload stores (negative control)
 PUBLISH_EARLY = 16
 CODES = {0: "passed", 1: "READY timeout", 2: "ACK timeout", 3: "the other side gave up", 4: "payload mismatch"}
