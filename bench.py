@@ -56,14 +56,14 @@ def build_inputs(tokens: int, topk: int, routing: str, heavy_tail: bool):
     return baseline_inputs(tokens, topk, routing, heavy_tail, WORLD, EXPERTS, HIDDEN)
 
 
-def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000, graph=False):
+def make_buffer(tokens, topk, wire, channels, fuse, timeout_ms=30000, graph=False, peer_threads=None):
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config = HostStagedConfig(channels=channels, stage=7 if wire == "fp8" else 6, wire_dtype="fp8_e4m3" if wire == "fp8" else "bf16",
                               fuse_receive_expand=fuse, receive_expand_mode="pipelined" if fuse else "scalar", timeout_ms=timeout_ms,
                               enable_graph=graph)
     return HostStagedEPBuffer(num_max_tokens_per_rank=tokens, hidden=HIDDEN, num_topk=topk, num_experts=EXPERTS, config=config,
-                              num_ranks=WORLD, rank=0, split_launch=SPLIT_LAUNCH)
+                              num_ranks=WORLD, rank=0, split_launch=SPLIT_LAUNCH, peer_threads=peer_threads)
 
 
 def set_peers(buffer, inputs):
@@ -116,12 +116,35 @@ def percentiles(values):
     return [pick(0.5), pick(0.95)]
 
 
+def source_stamp() -> str:
+    """Hash of the kernel sources the library was built from (csrc/*.hip, *.h,
+    *.cpp): every counter summary under profiles/ names the stamp of the sources it
+    was measured on, and a counted figure is only reported beside a live
+    measurement while the two agree."""
+    import hashlib
+
+    digest = hashlib.sha256()
+    for path in sorted((ROOT / "pcie-ep_amd" / "csrc").iterdir()):
+        if path.suffix in (".hip", ".h", ".cpp"):
+            digest.update(path.name.encode())
+            digest.update(path.read_bytes())
+    return digest.hexdigest()[:16]
+
+
+def stamped(summary: Path) -> bool:
+    """Whether a counter summary was measured on the sources of this build."""
+    for line in summary.read_text().splitlines():
+        if line.startswith("sources:"):
+            return line.split(":", 1)[1].strip().split()[0] == source_stamp()
+    return False
+
+
 def counted_traffic(tokens, topk, routing, wire):
     """HBM bytes per launch of the expand kernel as counted by rocprofv3 (FETCH_SIZE
     + WRITE_SIZE, scaled by the calibration copy), from the committed counter
     summary of exactly this workload; None when there is none."""
     summary = ROOT / "profiles" / f"expand_kernel_T{tokens}_top{topk}_{routing}_counters.txt"
-    if wire != "bf16" or not summary.exists():
+    if wire != "bf16" or not summary.exists() or not stamped(summary):
         return None
     for line in summary.read_text().splitlines():
         if line.startswith("hbm_traffic_bytes_per_launch"):
@@ -135,7 +158,7 @@ def counted_host_traffic(tokens, topk, routing, wire):
     copy), from the committed counter summary of exactly this workload."""
     summary = ROOT / "profiles" / f"transport_kernel_T{tokens}_top{topk}_{routing}_{wire}_counters.txt"
     found = {"read": None, "write": None}
-    if summary.exists():
+    if summary.exists() and stamped(summary):
         for line in summary.read_text().splitlines():
             for direction in found:
                 if line.startswith(f"host_{direction}_traffic_bytes_per_launch"):
@@ -211,14 +234,19 @@ def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, ver
 
     from helpers import verify_dispatch
 
-    buffer = make_buffer(tokens, topk, wire, channels, fuse=True)
+    # Restaging, the host threads move as many bytes as the GPU: every peer's source and receiver get a thread each.
+    buffer = make_buffer(tokens, topk, wire, channels, fuse=True, peer_threads=2 * (WORLD - 1) if restage else None)
     try:
         sizes = buffer.runtime.sizes
         payload_bytes, meta_bytes = int(sizes.payload_bytes), int(sizes.meta_bytes)
         set_peers(buffer, inputs)
         x, idx, weights = (item.cuda() for item in inputs[0])
-        buffer.peers.start(warmup + 2 * steps + (1 if verify else 0), restage=restage, read_rows=restage)
+        sync_steps = steps if tokens <= 512 else 0
+        stage_started = time.perf_counter()
+        buffer.peers.start(warmup + 3 * steps + sync_steps + (1 if verify else 0), restage=restage, read_rows=restage)
         buffer.peers.wait_staged(120_000)
+        # The emulator on its own: the first epoch is staged while the GPU is idle.
+        stage_seconds = time.perf_counter() - stage_started
         for _ in range(warmup):
             result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
             del result
@@ -231,6 +259,30 @@ def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, ver
             del result
         torch.cuda.synchronize()
         ms_per_step = (time.perf_counter() - started) / steps * 1e3
+
+        # The reference harness's figure (benchmarks/benchmark.py:165-198): an event pair
+        # around every whole dispatch, on the stream the dispatch runs on.
+        comm = buffer.get_comm_stream()
+        pairs = []
+        for _ in range(steps):
+            before, after = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            before.record(comm)
+            result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
+            after.record(comm)
+            pairs.append((before, after))
+            del result
+        torch.cuda.synchronize()
+        event_us = [before.elapsed_time(after) * 1e3 for before, after in pairs]
+        # The default, synchronous mode (the caller's stream waits for every result) at
+        # the sizes where the submission cost shows.
+        sync_us = None
+        if sync_steps:
+            started = time.perf_counter()
+            for _ in range(sync_steps):
+                result = buffer.dispatch(x, idx, weights, do_expand=True)
+                del result
+            torch.cuda.synchronize()
+            sync_us = (time.perf_counter() - started) / sync_steps * 1e6
 
         # Per-kernel durations: a second pass with HIP events recorded on the launch
         # stream around every kernel (reading them waits for that dispatch, so this
@@ -288,7 +340,10 @@ def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, ver
         "frac": read_bytes / (transport_ms * 1e-3) / 1e9 / h2d,
         "algorithmic_read_bytes": read_bytes, "algorithmic_write_bytes": write_bytes,
     }
+    event_stats = {"mean": mean(event_us), "p50": percentiles(event_us)[0], "p95": percentiles(event_us)[1]}
     return {
+        "dispatch_event_us": event_stats, "dispatch_sync_us": sync_us,
+        "emulator_stage_GBps": remote_reads * (payload_bytes + meta_bytes) / stage_seconds / 1e9 if restage else None,
         "ms_per_step": ms_per_step, "kernel_ms": kernel_ms, "pcie": pcie, "parity": parity, "payload_bytes": payload_bytes,
         "value": (own_writes + remote_reads) * payload_bytes / (ms_per_step * 1e-3) / 1e9,
         "rows": {"own_published": own_writes, "remote_unique": remote_reads, "local_unique": unique - remote_reads, "expanded": expanded},
@@ -301,6 +356,7 @@ def compact(run, tokens, topk):
     return {
         "dispatch_us": run["ms_per_step"] * 1e3, "transport_us": mean(run["kernel_ms"]["transport"]) * 1e3,
         "prologue_us": mean(run["kernel_ms"]["prologue"]) * 1e3, "payload_GBps": run["value"],
+        "dispatch_event_us": run["dispatch_event_us"], "dispatch_sync_us": run["dispatch_sync_us"],
         "pcie": run["pcie"]["frac"], "read_GBps": run["pcie"]["read_GBps"], "rows": run["rows"], "parity": run["parity"],
         "logical_GBps": tokens * topk * HIDDEN * 2 / (run["ms_per_step"] * 1e-3) / 1e9,
     }
@@ -395,6 +451,7 @@ def main() -> int:
                              "graph-replay / restaged sub-records); what the profiler runs use")
     parser.add_argument("--expand-only", action="store_true",
                         help="run only the calibration copy kernel and the stand-alone expand kernel (short; for counter collection)")
+    parser.add_argument("--source-stamp", action="store_true", help="print the hash of the kernel sources (the stamp of a profile summary) and exit")
     parser.add_argument("--split-launch", action="store_true",
                         help="run the prologue as a kernel of its own in front of the transport kernel (default: one launch per dispatch "
                              "wherever the prologue fits into the transport launch)")
@@ -404,6 +461,9 @@ def main() -> int:
     args = parser.parse_args()
     global SPLIT_LAUNCH
     SPLIT_LAUNCH = args.split_launch
+    if args.source_stamp:
+        print(source_stamp())
+        return 0
     if args.role_timeline:
         os.environ["PCIE_EP_PROFILING"] = "1"
     if args.gpus != 1:
@@ -451,18 +511,22 @@ def main() -> int:
     ms_per_step, kernel_ms, pcie = run["ms_per_step"], run["kernel_ms"], run["pcie"]
     traffic = counted_host_traffic(tokens, topk, args.routing, args.wire)
     pcie["traffic_read"], pcie["traffic_write"] = traffic["read"], traffic["write"]
+    if traffic["read"] is None:
+        pcie["traffic_note"] = "no counter summary under profiles/ carries the stamp of these kernel sources (" + source_stamp() + ")"
     record = {
         "metric": "dispatch PCIe payload GB/s ((U+F_r)*B/t) and us per dispatch, receiver rank 0 of 8",
         "value": run["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.wire == "bf16" else "fp8_e4m3 wire / bf16",
         "data": "synthetic",
+        "sources": source_stamp(),
         "config": {
             "workload": f"T={tokens}/source x 8 logical ranks, h{HIDDEN}, top-{topk} {args.routing}, {EXPERTS} experts (32 local), "
                         f"{args.wire} wire, C{args.channels}, Q=L=256, expand on, own TX + 7 host-staged sources",
             "tokens_per_rank": tokens, "hidden": HIDDEN, "topk": topk, "experts": EXPERTS, "channels": args.channels, "wire": args.wire,
-            "peer_restage": False,
+            "peer_restage": False, "launches_per_dispatch": 2 if SPLIT_LAUNCH else 1,
         },
-        "dispatch_us": ms_per_step * 1e3, "dispatch_gpu_us": (mean(kernel_ms["transport"]) + mean(kernel_ms["prologue"])) * 1e3,
+        "dispatch_us": ms_per_step * 1e3, "dispatch_event_us": run["dispatch_event_us"], "dispatch_sync_us": run["dispatch_sync_us"],
+        "dispatch_gpu_us": (mean(kernel_ms["transport"]) + mean(kernel_ms["prologue"])) * 1e3,
         "kernel_us": {name: mean(values) * 1e3 for name, values in kernel_ms.items()},
         "dispatch_gpu_us_p50_p95": percentiles([1e3 * sum(step) for step in zip(*kernel_ms.values())]),
         "pcie_pct_of_peak": 100.0 * pcie["frac"],
@@ -476,6 +540,8 @@ def main() -> int:
         record["roofline"] = measure_expand(inputs, tokens, topk, args.channels)
         record["roofline"]["hbm_copy_GBps"] = copy_rate.value
         record["roofline"]["traffic"] = counted_traffic(tokens, topk, args.routing, args.wire)
+        if record["roofline"]["traffic"] is None:
+            record["roofline"]["traffic_note"] = "no counter summary under profiles/ carries the stamp of these kernel sources (" + source_stamp() + ")"
     else:
         record["roofline"] = None
     if not args.skip_cpu_baseline:
@@ -493,8 +559,10 @@ def main() -> int:
         log("[bench] headline workload, peers restaging every step")
         restaged = run_workload(inputs, tokens, topk, args.wire, args.channels, max(3, steps // 4), 2, peaks, verify=False, restage=True)
         record["restaged"] = {"dispatch_us": restaged["ms_per_step"] * 1e3, "transport_us": mean(restaged["kernel_ms"]["transport"]) * 1e3,
-                              "pcie": restaged["pcie"]["frac"], "peer_restage": True,
-                              "note": "every source slot rewritten and every sent row read by the host threads per step; bounded by their staging rate"}
+                              "pcie": restaged["pcie"]["frac"], "read_GBps": restaged["pcie"]["read_GBps"], "peer_restage": True,
+                              "emulator_stage_GBps": restaged["emulator_stage_GBps"],
+                              "note": "every source slot rewritten and every sent row read by the host threads per step; "
+                                      "emulator_stage_GBps is their staging rate for the first epoch, with the GPU idle"}
         uniform_8192 = inputs if (tokens, args.routing, args.wire) == (8192, "uniform", "bf16") else None
         del inputs
         log("[bench] fp8 wire, heavy-tailed inputs, T=8192 top-8")

@@ -309,7 +309,8 @@ int pcie_ep_graph_launch(void* graph_exec, void* stream);
 /* Per-kernel timing with HIP events recorded on the dispatch stream (off by
  * default; must stay off for a dispatch that is being captured into a graph).
  * pcie_ep_get_kernel_times waits for the last timed dispatch and returns the
- * milliseconds of {prologue, transport, separate expand or 0}.
+ * milliseconds of {prologue, transport, separate expand or 0}; the prologue reads 0
+ * where it rides in the transport launch (the default wherever it fits).
  * No counterpart in the reference (its harness wraps events around the whole
  * dispatch: benchmarks/benchmark.py:165-198). */
 int pcie_ep_set_kernel_timing(pcie_ep_runtime* runtime, int32_t enable);

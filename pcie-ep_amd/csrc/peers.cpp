@@ -130,13 +130,17 @@ PeerEmulator::PeerEmulator(const SegmentLayout& layout, int local_rank, char* co
         state.expected.assign(channels, 0);
         state.consumed.assign(channels, 0);
     }
+    // A rank's two roles share no state, so they may run on different threads:
+    // the tasks are the peers' source roles followed by their receiver roles,
+    // dealt round; up to one thread per peer a rank's roles meet on one thread.
     const int peers = z_.dims.num_ranks - 1;
-    if (threads > peers) threads = peers;
+    if (threads > 2 * peers) threads = 2 * peers;
     if (threads < 1) threads = 1;
     assignment_.resize(threads);
     int next = 0;
-    for (int rank = 0; rank < z_.dims.num_ranks; ++rank)
-        if (rank != me_) assignment_[next++ % threads].push_back(rank);
+    for (int role : {kSourceRole, kReceiverRole})
+        for (int rank = 0; rank < z_.dims.num_ranks; ++rank)
+            if (rank != me_) assignment_[next++ % threads].push_back({rank, role});
     thread_done_.assign(threads, 0);
     for (int index = 0; index < threads; ++index) threads_.emplace_back([this, index] { thread_main(index); });
 }
@@ -275,18 +279,21 @@ void PeerEmulator::thread_main(int index) {
 
 bool PeerEmulator::serve_epoch(int index, uint64_t epoch, std::string& error) {
     const auto& mine = assignment_[index];
-    for (int rank : mine) {
-        Rank& state = ranks_[rank];
-        state.source_phase = 0;
-        state.receiver_phase = 0;
-        std::fill(state.cursor.begin(), state.cursor.end(), 0);
-        std::fill(state.sent.begin(), state.sent.end(), 0);
-        std::fill(state.consumed.begin(), state.consumed.end(), 0);
-        for (int slot_index : state.pending_slots) {
-            state.pending_sequence[slot_index] = 0;
-            state.pending_listed[slot_index] = 0;
+    for (const Task& task : mine) {
+        Rank& state = ranks_[task.rank];
+        if (task.role == kSourceRole) {
+            state.source_phase = 0;
+            std::fill(state.cursor.begin(), state.cursor.end(), 0);
+            std::fill(state.sent.begin(), state.sent.end(), 0);
+            for (int slot_index : state.pending_slots) {
+                state.pending_sequence[slot_index] = 0;
+                state.pending_listed[slot_index] = 0;
+            }
+            state.pending_slots.clear();
+            continue;
         }
-        state.pending_slots.clear();
+        state.receiver_phase = 0;
+        std::fill(state.consumed.begin(), state.consumed.end(), 0);
         state.receive_total = state.receive_done = 0;
         if (flags_ & kPeerCapture) {
             state.cap_tokens.clear(); state.cap_rank_ordinals.clear(); state.cap_expert_idx.clear();
@@ -294,29 +301,28 @@ bool PeerEmulator::serve_epoch(int index, uint64_t epoch, std::string& error) {
             state.cap_weights.clear(); state.cap_masks.clear();
         }
     }
-    std::vector<char> source_done(mine.size(), 0), receiver_done(mine.size(), 0);
+    std::vector<char> task_done(mine.size(), 0);
     double last_progress = now_seconds();
     while (true) {
         bool progressed = false, all_done = true;
         for (size_t i = 0; i < mine.size(); ++i) {
-            const int rank = mine[i];
-            if (!source_done[i]) {
-                bool done = false, quiescent = false;
+            if (task_done[i]) continue;
+            const int rank = mine[i].rank;
+            bool done = false;
+            if (mine[i].role == kSourceRole) {
+                bool quiescent = false;
                 progressed |= source_progress(rank, epoch, done, quiescent, error);
                 if (!error.empty()) return false;
                 if (done || quiescent) {
                     uint64_t seen = ranks_[rank].staged_epoch.load(std::memory_order_relaxed);
                     if (seen < epoch) ranks_[rank].staged_epoch.store(epoch, std::memory_order_release);
                 }
-                source_done[i] = done;
-            }
-            if (!receiver_done[i]) {
-                bool done = false;
+            } else {
                 progressed |= receiver_progress(rank, epoch, done, error);
                 if (!error.empty()) return false;
-                receiver_done[i] = done;
             }
-            all_done &= source_done[i] && receiver_done[i];
+            task_done[i] = done;
+            all_done &= done;
         }
         if (all_done) return true;
         if (cancel_.load() || failed_.load()) return false;
@@ -325,11 +331,14 @@ bool PeerEmulator::serve_epoch(int index, uint64_t epoch, std::string& error) {
             if (now_seconds() - last_progress > timeout_ms_ * 1e-3) {
                 std::string detail;
                 for (size_t i = 0; i < mine.size(); ++i) {
-                    const Rank& state = ranks_[mine[i]];
-                    detail += " rank " + std::to_string(mine[i]) + ": source phase " + std::to_string(state.source_phase) +
-                              (source_done[i] ? " done" : "") + ", receiver phase " + std::to_string(state.receiver_phase) +
-                              " (" + std::to_string(state.receive_done) + "/" + std::to_string(state.receive_total) + ")" +
-                              (receiver_done[i] ? " done;" : ";");
+                    const Rank& state = ranks_[mine[i].rank];
+                    if (mine[i].role == kSourceRole)
+                        detail += " rank " + std::to_string(mine[i].rank) + ": source phase " + std::to_string(state.source_phase) +
+                                  (task_done[i] ? " done;" : ";");
+                    else
+                        detail += " rank " + std::to_string(mine[i].rank) + ": receiver phase " + std::to_string(state.receiver_phase) + " (" +
+                                  std::to_string(state.receive_done) + "/" + std::to_string(state.receive_total) + ")" +
+                                  (task_done[i] ? " done;" : ";");
                 }
                 error = "peer emulator made no progress for " + std::to_string(timeout_ms_) + " ms in epoch " + std::to_string(epoch) + ":" + detail;
                 return false;

@@ -102,6 +102,10 @@ private:
         std::atomic<uint64_t> staged_epoch{0};
     };
 
+    // One role of one emulated rank: the unit of work a thread is given.
+    enum Role : int { kSourceRole = 0, kReceiverRole = 1 };
+    struct Task { int rank; int role; };
+
     void thread_main(int index);
     bool serve_epoch(int index, uint64_t epoch, std::string& error);
     bool source_progress(int rank, uint64_t epoch, bool& done, bool& quiescent, std::string& error);
@@ -119,7 +123,7 @@ private:
     int timeout_ms_;
     std::vector<Rank> ranks_;
     std::vector<std::thread> threads_;
-    std::vector<std::vector<int>> assignment_;
+    std::vector<std::vector<Task>> assignment_;
     std::vector<uint64_t> thread_done_;  // epochs completed per thread (under mutex_)
     std::mutex mutex_;
     std::condition_variable wake_, finished_;

@@ -260,6 +260,7 @@ struct pcie_ep_runtime {
     bool timing = false;
     bool timing_valid = false;
     bool timing_expand = false;
+    bool timing_split = false;  // the timed dispatch ran the prologue as a kernel of its own
     hipEvent_t marks[4] = {};
     // Recorded behind every dispatch through the static scratch (created with the runtime:
     // that entry point must not allocate).
@@ -661,7 +662,8 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     rt->timing_valid = false;
     if (timed) HIP_TRY(hipEventRecord(rt->marks[0], stream));
     if (!state.fused) HIP_TRY(launch_prologue(state, stream));
-    if (timed) HIP_TRY(hipEventRecord(rt->marks[1], stream));
+    // One launch per dispatch: the prologue rides in the transport launch and has no span of its own.
+    if (timed && !state.fused) HIP_TRY(hipEventRecord(rt->marks[1], stream));
     HIP_TRY(launch_transport(state, stream));
     if (timed) HIP_TRY(hipEventRecord(rt->marks[2], stream));
     const bool separate_expand = state.expand && !state.fuse_expand;
@@ -669,6 +671,7 @@ int pcie_ep_dispatch(pcie_ep_runtime* rt, const pcie_ep_dispatch_args* args, voi
     if (timed) {
         HIP_TRY(hipEventRecord(rt->marks[3], stream));
         rt->timing_expand = separate_expand;
+        rt->timing_split = !state.fused;
         rt->timing_valid = true;
     }
     return 0;
@@ -786,8 +789,8 @@ int pcie_ep_get_kernel_times(pcie_ep_runtime* rt, float* milliseconds) {
     if (!rt->timing_valid) return set_error(PCIE_EP_E_STATE, "no timed dispatch has been recorded");
     HIP_TRY(hipEventSynchronize(rt->marks[3]));
     milliseconds[0] = milliseconds[1] = milliseconds[2] = 0.0f;
-    HIP_TRY(hipEventElapsedTime(milliseconds + 0, rt->marks[0], rt->marks[1]));
-    HIP_TRY(hipEventElapsedTime(milliseconds + 1, rt->marks[1], rt->marks[2]));
+    if (rt->timing_split) HIP_TRY(hipEventElapsedTime(milliseconds + 0, rt->marks[0], rt->marks[1]));
+    HIP_TRY(hipEventElapsedTime(milliseconds + 1, rt->marks[rt->timing_split ? 1 : 0], rt->marks[2]));
     if (rt->timing_expand) HIP_TRY(hipEventElapsedTime(milliseconds + 2, rt->marks[2], rt->marks[3]));
     return 0;
 }

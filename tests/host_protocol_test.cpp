@@ -106,6 +106,7 @@ int check_captured(PeerEmulator& emulator, int receiver, const Inputs& sent, int
 int main(int argc, char** argv) {
     const bool relay = argc > 1 && std::string(argv[1]) == "relay";
     const int epochs = argc > 2 ? std::atoi(argv[2]) : 4;
+    const int threads = argc > 3 ? std::atoi(argv[3]) : 1;  // 2: the peer's source and receiver roles on a thread each
     Dimensions dims{kRanks, kTokens, kHidden, kTopk, kExperts, kChannels, /*payload_slots*/ 2, /*descriptor_slots*/ 1, /*wire_fp8*/ 0};
     if (relay) {
         dims.domains = 2;
@@ -125,8 +126,8 @@ int main(int argc, char** argv) {
     options.pin = false;
     int status = 0;
     {
-        PeerEmulator gpu_is_rank0(z, 0, segments, replica, 1, 20000, options);  // runs rank 1
-        PeerEmulator gpu_is_rank1(z, 1, segments, replica, 1, 20000, options);  // runs rank 0
+        PeerEmulator gpu_is_rank0(z, 0, segments, replica, threads, 20000, options);  // runs rank 1
+        PeerEmulator gpu_is_rank1(z, 1, segments, replica, threads, 20000, options);  // runs rank 0
         std::string error;
         for (int epoch = 0; epoch < epochs && !status; ++epoch) {
             // Token counts change from epoch to epoch, including an empty source.

@@ -39,3 +39,26 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-9
     baseline = record["cpu_baseline"]
     assert baseline["kind"] == "port" and baseline["cores"] >= 1 and baseline["value"] > 0 and baseline["sample"]
+    # The reference harness's own measure (an event pair around each whole dispatch) and the default synchronous mode.
+    events = record["dispatch_event_us"]
+    assert 0 < events["p50"] <= events["p95"] and events["mean"] > 0
+    assert record["dispatch_sync_us"] > 0  # reported up to 512 tokens, where the submission cost shows
+    # A counted figure is reported only with a summary measured on these kernel sources; otherwise null, with a note.
+    assert len(record["sources"]) == 16
+    assert "traffic" in roofline and (roofline["traffic"] is not None or "traffic_note" in roofline)
+    assert record["pcie"]["traffic_read"] is not None or "traffic_note" in record["pcie"]
+
+
+def test_counter_summaries_are_stamped_with_the_sources_they_were_measured_on():
+    """Every counted figure bench.py may quote comes from a summary that names the
+    hash of the kernel sources it was measured on and the command that made it."""
+    sys.path.insert(0, str(ROOT))
+    import bench
+
+    stamp = bench.source_stamp()
+    assert len(stamp) == 16 and stamp == bench.source_stamp()
+    for summary in sorted((ROOT / "profiles").glob("*.txt")):
+        text = summary.read_text()
+        assert any(line.startswith("sources:") for line in text.splitlines()), summary.name
+        assert any(line.startswith("command") for line in text.splitlines()), summary.name
+

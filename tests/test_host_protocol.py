@@ -35,9 +35,11 @@ def program(request, tmp_path_factory):
     return binary
 
 
+@pytest.mark.parametrize("threads", [1, 2])
 @pytest.mark.parametrize("mode", ["direct", "relay"])
-def test_two_emulators_exchange_rows(program, mode):
-    outcome = subprocess.run([str(program), mode, "6"], capture_output=True, text=True, timeout=300)
+def test_two_emulators_exchange_rows(program, mode, threads):
+    """``threads=2`` runs the peer's source and receiver roles on a thread each."""
+    outcome = subprocess.run([str(program), mode, "6", str(threads)], capture_output=True, text=True, timeout=300)
     report = outcome.stdout[-2000:] + outcome.stderr[-4000:]
     assert outcome.returncode == 0, report
     assert "host protocol test passed" in outcome.stdout, report
