@@ -1,6 +1,7 @@
 // E4M3FN wire arithmetic shared by the gfx950 kernels and the host peer
-// emulator.  Everything is integer ALU on FP32 bit patterns so that the GPU
-// and the CPU produce the same bytes:
+// emulator.  The host side is integer ALU on FP32 bit patterns; the kernels use
+// gfx950's conversion instructions (OCP E4M3FN <-> FP32, FP32 -> BF16, all round
+// to nearest even), which produce the same bytes for every finite input:
 //   scale  = amax == 0 ? 1 : max(amax / 448, 2^-126)
 //   code   = e4m3_rne_satfinite(clamp(x * (1 / scale), -448, 448))
 //   decode = bf16_rne(float(e4m3(code)) * scale)
@@ -45,9 +46,22 @@ PCIE_EP_FP8_HD float bf16_to_float(uint16_t bits) { return bits_float(uint32_t(b
 
 // Round to nearest even; inputs are finite.
 PCIE_EP_FP8_HD uint16_t float_to_bf16_rne(float value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(value));
+#else
     const uint32_t raw = float_bits(value);
     return uint16_t((raw + 0x7FFFu + ((raw >> 16) & 1u)) >> 16);
+#endif
 }
+#if defined(__HIPCC__)
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// Two FP32 -> two BF16 in one word (first element in the low half), one instruction.
+__device__ __forceinline__ uint32_t float2_to_bf16x2_rne(float first, float second) {
+    const f32x2 pair = {first, second};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+}
+#endif
 
 PCIE_EP_FP8_HD float fp8_scale_from_amax(float amax) {
     if (amax == 0.0f) return 1.0f;
@@ -57,6 +71,10 @@ PCIE_EP_FP8_HD float fp8_scale_from_amax(float amax) {
 
 // FP32 -> E4M3FN, round to nearest even, finite values saturate to 0x7E.
 PCIE_EP_FP8_HD uint8_t e4m3_encode(float value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // |value| <= 448 or NaN here (the caller clamps): nothing for the instruction to saturate.
+    return uint8_t(__builtin_amdgcn_cvt_pk_fp8_f32(value, 0.0f, 0, false));
+#endif
     const uint32_t raw = float_bits(value);
     const uint32_t sign = (raw >> 24) & 0x80u;
     const uint32_t magnitude = raw & 0x7FFFFFFFu;
@@ -87,6 +105,10 @@ PCIE_EP_FP8_HD uint8_t e4m3_encode(float value) {
 
 // E4M3FN -> FP32, exact.
 PCIE_EP_FP8_HD float e4m3_decode(uint8_t code) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_cvt_f32_fp8(int(code), 0);
+#endif
+    if ((code & 0x7Fu) == 0x7Fu) return bits_float(0x7FC00000u);  // NaN (outside the wire contract)
     const uint32_t sign = uint32_t(code & 0x80u) << 24;
     const uint32_t exponent = (code >> 3) & 0xFu;
     const uint32_t mantissa = code & 0x7u;
@@ -107,5 +129,23 @@ PCIE_EP_FP8_HD uint8_t fp8_quantize_element(uint16_t bf16_bits, float inverse_sc
 PCIE_EP_FP8_HD uint16_t fp8_dequantize_element(uint8_t code, float scale) {
     return float_to_bf16_rne(e4m3_decode(code) * scale);
 }
+
+#if defined(__HIPCC__)
+__device__ __forceinline__ float fp8_clamp(float scaled) { return scaled > kE4M3Max ? kE4M3Max : (scaled < -kE4M3Max ? -kE4M3Max : scaled); }
+// Four BF16 (two words, elements in order) -> four codes in one word.
+__device__ __forceinline__ uint32_t fp8_quantize_word(uint32_t first, uint32_t second, float inverse_scale) {
+    const float a = fp8_clamp(bits_float(first << 16) * inverse_scale), b = fp8_clamp(bits_float(first & 0xFFFF0000u) * inverse_scale);
+    const float c = fp8_clamp(bits_float(second << 16) * inverse_scale), d = fp8_clamp(bits_float(second & 0xFFFF0000u) * inverse_scale);
+    int codes = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    codes = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, codes, true);
+    return uint32_t(codes);
+}
+// Four codes of one word -> four BF16 (two words, elements in order).
+__device__ __forceinline__ void fp8_dequantize_word(uint32_t codes, float scale, uint32_t& first, uint32_t& second) {
+    const f32x2 low = __builtin_amdgcn_cvt_pk_f32_fp8(int(codes), false), high = __builtin_amdgcn_cvt_pk_f32_fp8(int(codes), true);
+    first = float2_to_bf16x2_rne(low[0] * scale, low[1] * scale);
+    second = float2_to_bf16x2_rne(high[0] * scale, high[1] * scale);
+}
+#endif
 
 }  // namespace pcie_ep

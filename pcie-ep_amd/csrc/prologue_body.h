@@ -66,6 +66,39 @@ struct ChunkRecord {
     __host__ __device__ int error_key() const { return chan_relay() + channels * domains; }
 };
 
+// Field-wise sums over `count` chunk records (record r begins at first + r * stride,
+// `fields` consecutive words of each are summed) into sums[fields] in LDS, by the
+// whole workgroup.  A read of another workgroup's record is a trip to memory of half
+// a microsecond: the (record, field) pairs are dealt round the threads and read
+// kBatch at a time, each batch issued back to back and waited for once, so the
+// trips overlap instead of following each other.
+template <int kBatch>
+__device__ __forceinline__ void sum_chunk_records(const int32_t* first, int stride, int fields, int count, int* sums) {
+    for (int field = threadIdx.x; field < fields; field += blockDim.x) sums[field] = 0;
+    lds_barrier();
+    const int total = fields * count, step = int(blockDim.x);
+    int record = int(threadIdx.x) / fields, field = int(threadIdx.x) % fields;
+    for (int n = threadIdx.x; n < total; n += step * kBatch) {
+        int value[kBatch], where[kBatch];
+#pragma unroll
+        for (int slot = 0; slot < kBatch; ++slot) {
+            const bool valid = n + slot * step < total;
+            where[slot] = valid ? field : -1;
+            // Past the end: a harmless read of the first word instead of a branch between the loads.
+            value[slot] = device_load_global(first + (valid ? size_t(record) * stride + field : size_t(0)));
+            field += step;
+            while (field >= fields) {
+                field -= fields;
+                ++record;
+            }
+        }
+#pragma unroll
+        for (int slot = 0; slot < kBatch; ++slot)
+            if (where[slot] >= 0 && value[slot] != 0) atomicAdd(sums + where[slot], value[slot]);
+    }
+    lds_barrier();
+}
+
 // The count mailboxes of every destination (layout.cuh:7-20) from the plan's
 // totals in LDS: host stores issued, not waited for.  A mailbox block starts on a
 // 128-byte line and is stored as whole 16-byte vectors (the words behind its last
@@ -470,14 +503,7 @@ __device__ __forceinline__ void prologue_chunk(const DeviceState& state, unsigne
                 }
             }
             __syncthreads();
-            if (!stalled && !leader) {
-                for (int bin = threadIdx.x; bin < bins; bin += blockDim.x) {
-                    int sum = 0;
-                    for (int earlier = 0; earlier < chunk; ++earlier)
-                        sum += device_load(chunk_records + size_t(earlier) * record.stride() + record.counts() + bin);
-                    base[bin] = sum;
-                }
-            }
+            if (!stalled && !leader) sum_chunk_records<16>(chunk_records + record.counts(), record.stride(), bins, chunk, base);
             __syncthreads();
         }
         PCIE_EP_PROFILE(profile.first(kPrologueChunkTotalsNs);)
@@ -572,6 +598,7 @@ __device__ __forceinline__ void prologue_chunk(const DeviceState& state, unsigne
             else totals[field] = state.plan_chan_relay[field - record.chan_relay()];
         }
     } else if (chunks != 1) {
+        if (!layout && threadIdx.x == 0) *first_error = 0x7FFFFFFF;  // nothing to lay out: no chunk has run
         for (int other = threadIdx.x; other < chunks; other += blockDim.x) {
             while (device_load(chunk_flags + other) != tag) {
                 if (now_ticks() - begin_ticks > state.timeout_ticks) {
@@ -583,17 +610,11 @@ __device__ __forceinline__ void prologue_chunk(const DeviceState& state, unsigne
         }
         __syncthreads();
         if (!stalled) {
-            for (int field = threadIdx.x; field < fields; field += blockDim.x) {
-                int sum = 0;
-                for (int other = 0; other < chunks; ++other) sum += device_load(chunk_records + size_t(other) * record.stride() + field);
-                totals[field] = sum;
-            }
-            if (threadIdx.x == 0) {
-                for (int other = 0; other < chunks; ++other) {
-                    const int candidate = device_load(chunk_records + size_t(other) * record.stride() + record.error_key());
-                    route_error = candidate < route_error ? candidate : route_error;
-                }
-            }
+            // The lowest error key of any chunk (the leader's own is in place already).
+            for (int other = threadIdx.x; other < chunks; other += blockDim.x)
+                atomicMin(first_error, device_load(chunk_records + size_t(other) * record.stride() + record.error_key()));
+            sum_chunk_records<32>(chunk_records, record.stride(), fields, chunks, totals);
+            route_error = *first_error;
         }
     }
     lds_barrier();

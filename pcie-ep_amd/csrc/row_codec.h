@@ -98,10 +98,7 @@ __device__ __forceinline__ float quantize_row(const uint16_t* input, const Sink&
             for (int word = 0; word < 4; ++word) {
                 const uint32_t a = word < 2 ? lo[word * 2] : hi[(word - 2) * 2];
                 const uint32_t b = word < 2 ? lo[word * 2 + 1] : hi[(word - 2) * 2 + 1];
-                codes[word] = uint32_t(fp8_quantize_element(uint16_t(a & 0xFFFFu), inverse)) |
-                              uint32_t(fp8_quantize_element(uint16_t(a >> 16), inverse)) << 8 |
-                              uint32_t(fp8_quantize_element(uint16_t(b & 0xFFFFu), inverse)) << 16 |
-                              uint32_t(fp8_quantize_element(uint16_t(b >> 16), inverse)) << 24;
+                codes[word] = fp8_quantize_word(a, b, inverse);
             }
             sink.vector(group, codes);
         }
@@ -116,8 +113,8 @@ __device__ __forceinline__ void dequantize_vector(const u32x4& codes, float scal
 #pragma unroll
     for (int word = 0; word < 4; ++word) {
         const uint32_t c = codes[word];
-        const uint32_t a = uint32_t(fp8_dequantize_element(uint8_t(c), scale)) | uint32_t(fp8_dequantize_element(uint8_t(c >> 8), scale)) << 16;
-        const uint32_t b = uint32_t(fp8_dequantize_element(uint8_t(c >> 16), scale)) | uint32_t(fp8_dequantize_element(uint8_t(c >> 24), scale)) << 16;
+        uint32_t a, b;
+        fp8_dequantize_word(c, scale, a, b);
         if (word < 2) {
             lo[word * 2] = a;
             lo[word * 2 + 1] = b;
