@@ -980,14 +980,19 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
         // Tickets are handed out from the first descriptor on, but no row is requested
         // before the producer of the prefixes has put its reads of the count mailboxes
         // on the link (a few hundred bytes that everything waits for must not queue
-        // behind megabytes of row reads) nor, with the prologue in the same launch,
-        // before the own counts are with the peers (their acknowledgement would).
+        // behind megabytes of row reads).  That producer has seen every source's counts by
+        // then.  The prologue of the same launch may still be laying out thousands of own
+        // tokens: count stores that leave with rows already in flight are acknowledged some
+        // 12 us later than on an idle link (measured), so a peer whose counts came early
+        // learns this rank's that much later.  It holds its first rows in registers for as
+        // long, with their requests on the link - no link time is lost - and among ranks
+        // that start together every gate opens after the last counts have arrived anyway.
         // The wavefront waits here with its ticket read and its addresses computed:
         // the requests leave the moment the gate opens.
         while (!gate_open) {
             int gate = 0;
             if (lane == 0) {
-                if ((device_load(state.receive_prefix_state) & kPrefixRequested) && (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch))) gate = 1;
+                if (device_load(state.receive_prefix_state) & kPrefixRequested) gate = 1;
                 else if (aborted(q) || device_load(state.receive_prefix_state + 1) == kPrefixFailed) gate = -1;
                 else if (deadline.expired(state)) {
                     record_error(state, kErrRingProgressWait);
@@ -1277,8 +1282,7 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
                 // wavefront did, they would all fire at once and each would have its first
                 // row after the time the link needs for all of them, with nobody left to transmit.
                 if (rx_backlog && !gate_seen && rx_head >= kPreGateRows) {
-                    gate_seen = (device_load(state.receive_prefix_state) & kPrefixRequested) &&
-                                (!state.fused || device_load(&q.plan_ready.value) == epoch_flag(epoch));
+                    gate_seen = (device_load(state.receive_prefix_state) & kPrefixRequested) != 0;
                     rx_backlog = gate_seen != 0;
                 }
                 const int tx_total = device_load(&q.tx_head.total), rx_total = device_load(&q.rx_head.total);
