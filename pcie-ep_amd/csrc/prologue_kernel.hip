@@ -1,7 +1,7 @@
 // Prologue kernel: the dispatch prologue (prologue_body.h) as a launch of its own,
 // one workgroup per chunk of up to 16 wavefronts of tokens, in front of the
 // transport kernel.  Used when the prologue cannot ride in the transport kernel's
-// launch (see launch_dispatch in transport_kernel.hip).
+// launch (the runtime decides at create time: `fused` in runtime.hip), or when the caller asks for it.
 #include "prologue_body.h"
 
 namespace pcie_ep {

@@ -92,7 +92,7 @@ int NumaRelay::diagnostics(RelayFlowRecord* records, int capacity) const {
             r.channel = flow->channel;
             r.domain = flow->domain;
             r.worker = int(w);
-            r.cpu = worker.cpu;
+            r.cpu = worker.cpu.load(std::memory_order_relaxed);
             r.epoch = flow->diagnostic_epoch.load(std::memory_order_acquire);
             r.expected_tokens = flow->diagnostic_expected.load(std::memory_order_relaxed);
             r.copied_tokens = flow->diagnostic_copies.load(std::memory_order_relaxed);
@@ -118,24 +118,30 @@ std::string NumaRelay::worker_errors() const {
 }
 
 // Pin the worker to one allowed CPU of its domain's node (numa_relay.hpp:178-199).
-// A node that does not exist on this machine leaves the worker unpinned.
+// A node that does not exist on this machine has no CPU list: the worker is then
+// pinned among the CPUs the caller asked for (relay_cpu_affinity) if there are any,
+// and left unpinned otherwise - the reference refuses such a map ("no allowed CPU on
+// requested relay NUMA node", numa_relay.hpp:192-206), which would rule out every
+// logical NUMA map on a one-node machine.  A request none of whose CPUs is allowed
+// fails as in the reference.
 void NumaRelay::pin(Worker& worker) {
     if (!options_.pin) return;
     const std::vector<int> node_cpus = numa_node_cpus(options_.domain_node[worker.domain]);
-    if (node_cpus.empty()) return;
+    if (node_cpus.empty() && options_.cpus.empty()) return;
     cpu_set_t allowed;
     CPU_ZERO(&allowed);
     if (pthread_getaffinity_np(pthread_self(), sizeof allowed, &allowed) != 0) throw std::runtime_error("cannot query relay thread CPU affinity");
     std::vector<int> candidates;
-    for (int cpu : node_cpus) {
+    for (int cpu : node_cpus.empty() ? options_.cpus : node_cpus) {
         const bool wanted = options_.cpus.empty() || std::find(options_.cpus.begin(), options_.cpus.end(), cpu) != options_.cpus.end();
         if (cpu >= 0 && cpu < CPU_SETSIZE && CPU_ISSET(cpu, &allowed) && wanted) candidates.push_back(cpu);
     }
     if (candidates.empty()) throw std::runtime_error("no allowed CPU on requested relay NUMA node");
-    worker.cpu = candidates[size_t(rank_ * options_.workers_per_domain + worker.index) % candidates.size()];
+    const int chosen = candidates[size_t(rank_ * options_.workers_per_domain + worker.index) % candidates.size()];
+    worker.cpu.store(chosen, std::memory_order_relaxed);
     cpu_set_t target;
     CPU_ZERO(&target);
-    CPU_SET(worker.cpu, &target);
+    CPU_SET(chosen, &target);
     if (const int status = pthread_setaffinity_np(pthread_self(), sizeof target, &target))
         throw std::runtime_error("cannot pin relay worker: " + std::to_string(status));
 }

@@ -91,7 +91,8 @@ private:
         Flow(int c, int n, int slots) : channel(c), domain(n), replica_sequences(slots, 0), replica_masks(slots, 0) {}
     };
     struct Worker {
-        int domain = 0, index = 0, cpu = -1;
+        int domain = 0, index = 0;
+        std::atomic<int> cpu{-1};  // written by the worker thread when it pins itself, read by diagnostics()
         std::string runtime_error;
         mutable std::mutex guard;
         std::vector<std::unique_ptr<Flow>> flows;

@@ -20,15 +20,27 @@
 //    from popcounts of ballots; RX control probes up to 64/P descriptors per
 //    source per iteration instead of one source per iteration.
 //  * Work is handed out through two global ticket rings in device memory (one
-//    for TX, one for RX).  Workgroup b < C is the control workgroup of channel
-//    b (TX control + RX control); the workgroups after them only hold payload
-//    wavefronts, which claim tickets of ANY channel.  Consecutive workgroup ids
-//    land on consecutive XCDs, so every channel's rows are moved by all eight
-//    XCDs.  This matters because the XCDs get unequal shares of the host link:
-//    with workers bound to their channel's workgroup, equal work finished in
-//    8.8 ms on the best XCD and 12.8 ms on the worst.  It also decouples the
-//    bytes in flight (worker wavefronts x row size), which set the latency of
-//    every control-path read, from the number of channels.
+//    for TX, one for RX).  Control wavefronts only reserve and hand out tickets;
+//    the payload workgroups hold payload wavefronts, which claim tickets of ANY
+//    channel, so every channel's rows are moved by all payload XCDs.  This matters
+//    because the XCDs get unequal shares of the host link: with workers bound to
+//    their channel's workgroup, equal work finished in 8.8 ms on the best XCD and
+//    12.8 ms on the worst.  It also decouples the bytes in flight (worker
+//    wavefronts x row size), which set the latency of every control-path read,
+//    from the number of channels.
+//  * Which workgroup runs on which XCD is chosen (workgroup id = row * 8 + XCD):
+//    two XCDs hold the control class - the epoch begin and the layout chunks of the
+//    prologue when it rides in this launch, and per pair of channels one workgroup
+//    of transmit controls and one of receive controls, on different XCDs - and six
+//    hold the payload class (payload and local-bypass workgroups).  A host read
+//    stays in its XCD's memory queues for as long as the link needs for the bytes
+//    requested before it, and every other memory operation through that XCD waits
+//    behind it: controls that shared an XCD with payload wavefronts saw their
+//    tickets and flags arrive tens of microseconds late.
+//  * With the prologue in the same launch (one launch per dispatch), the roles
+//    here start with the queues not yet reset: one thread per workgroup waits for
+//    the epoch begin's word before its role touches them, the transmit side and
+//    the local bypass wait for the plan's word, the receive side for neither.
 //  * Workers publish their own descriptors and payload ACKs as soon as their own
 //    stores / loads have completed; control wavefronts only reserve and hand out.
 //  * A payload wavefront has no fixed direction: before every row it takes the

@@ -44,3 +44,27 @@ def test_two_emulators_exchange_rows(program, mode, threads):
     assert outcome.returncode == 0, report
     assert "host protocol test passed" in outcome.stdout, report
     assert "Sanitizer" not in outcome.stderr, report
+
+
+@pytest.fixture(scope="module", params=sorted(SANITIZERS))
+def relay_program(request, tmp_path_factory):
+    if shutil.which("g++") is None:
+        pytest.skip("no host compiler")
+    binary = tmp_path_factory.mktemp("relay_failure") / f"relay_failure_{request.param}"
+    command = ["g++", "-std=c++20", "-O1", "-g", "-fno-omit-frame-pointer", SANITIZERS[request.param], "-fno-sanitize-recover=all", "-pthread",
+               f"-I{CSRC}", str(ROOT / "tests" / "relay_failure_test.cpp"), str(CSRC / "relay.cpp"), "-o", str(binary)]
+    built = subprocess.run(command, capture_output=True, text=True, timeout=600)
+    assert built.returncode == 0, built.stderr[-3000:]
+    return binary
+
+
+def test_relay_failure_paths(relay_program):
+    """One relay on a hand-built segment: a pinned happy path, the failure codes
+    101-106 (epoch changed before the drain, timeout, slot outside the ring,
+    identity mismatch, no destination in the domain, worker exception) and the
+    stickiness of a failed flow; the worker threads join in every case."""
+    outcome = subprocess.run([str(relay_program)], capture_output=True, text=True, timeout=300)
+    report = outcome.stdout[-2000:] + outcome.stderr[-4000:]
+    assert outcome.returncode == 0, report
+    assert "relay failure test passed" in outcome.stdout, report
+    assert "Sanitizer" not in outcome.stderr, report
