@@ -276,6 +276,12 @@ enum ProfileField : int {
     kProfileRxPrefixWaitSum,     // sampled: waiting for the receive prefixes (first rows only)
     kProfileRxScatterSum,        // sampled: row loads issued -> destination rows' stores issued
     kProfileGateOpenNs,          // first received row: the gate in front of the row requests seen open
+    // The way of this wavefront's first row, as points in time:
+    kProfileFirstLookNs,         // the look at the queues that found the row's ticket
+    kProfileFirstTaggedNs,       // ticket claimed and its tag seen ready
+    kProfileFirstEntryNs,        // ticket entry read (receive side)
+    kProfileFirstRequestNs,      // metadata and first payload loads issued (receive side)
+    kProfileFirstDataNs,         // metadata back (receive side)
 };
 // Record of the prologue's leader workgroup (thread 0), stored behind the payload wavefronts' records.
 enum PrologueProfileField : int {

@@ -979,6 +979,7 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
         const uint64_t payload_sequence = uint64_t(uint32_t(__shfl(int(word), 4))) | uint64_t(uint32_t(__shfl(int(word), 5))) << 32;
         const int channel_ordinal = __shfl(int(word), 6);
         const bool replica = __shfl(int(word), 7) != 0;
+        PCIE_EP_PROFILE(profile.first(kProfileFirstEntryNs);)
         // The ticket now lives in registers: its ring entry may be reused while
         // this wavefront is still moving the row.
         wait_memory_ops();
@@ -1042,6 +1043,7 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
                 for (int j = 0; j < kPassItems; ++j) row.v[j] = host_load_b128(payload, uint32_t(j * kWave + lane) * 16u);
             }
         }
+        PCIE_EP_PROFILE(profile.first(kProfileFirstRequestNs);)
         if (lane < kScratchDwords / 4) {
             scratch[lane * 4] = meta_vector[0];
             scratch[lane * 4 + 1] = meta_vector[1];
@@ -1049,6 +1051,7 @@ __device__ __forceinline__ bool rx_row(const DeviceState& state, TransportQueues
             scratch[lane * 4 + 3] = meta_vector[3];
         }
         fence_lds();
+        PCIE_EP_PROFILE(profile.first(kProfileFirstDataNs);)
         const int token = int(scratch[0]);
         const float scale = bits_float(scratch[2]);
         if (token != ticket_token || payload_sequence != sequence(epoch, token)) {
@@ -1281,6 +1284,7 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
     while (true) {
         // 0: nothing to do now, 1: transmit, 2: receive, -1: both directions are finished or the kernel aborts.
         int choice = 0;
+        PCIE_EP_PROFILE(const uint64_t look_begin = profile.now();)
         int gate_seen = gate_open ? 1 : 0;
         if (lane == 0) {
             if (aborted(q)) choice = -1;
@@ -1347,7 +1351,7 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
         PCIE_EP_PROFILE(if (idle_begin) { profile.add(kProfileIdleSum, profile.now() - idle_begin); idle_begin = 0; })
         const bool transmit = choice == 1;
         QueueCounter& head = transmit ? q.tx_head : q.rx_head;
-        PCIE_EP_PROFILE(profile.first(kProfileFirstClaimNs); const uint64_t claim_begin = profile.now();)
+        PCIE_EP_PROFILE(profile.first(kProfileFirstClaimNs); const uint64_t claim_begin = profile.now(); if (!profile.values[kProfileFirstLookNs]) profile.values[kProfileFirstLookNs] = look_begin;)
         const int ticket_index = claim_ticket(head, lane);
         // Several wavefronts may have seen the same backlog: a claim beyond the last
         // ticket of the dispatch is simply dropped, an earlier one waits for its tag.
@@ -1355,7 +1359,7 @@ __device__ __forceinline__ void payload_worker(const DeviceState& state, Transpo
             if (broadcast_first(aborted(q) ? 1 : 0)) break;
             continue;
         }
-        PCIE_EP_PROFILE(profile.add(kProfileTicketWaitSum, profile.now() - claim_begin); const bool sampled = rows_moved++ % kProfileSampleStride == 0;
+        PCIE_EP_PROFILE(profile.first(kProfileFirstTaggedNs); profile.add(kProfileTicketWaitSum, profile.now() - claim_begin); const bool sampled = rows_moved++ % kProfileSampleStride == 0;
                         if (sampled) profile.add(transmit ? kProfileSampledTxRows : kProfileSampledRxRows); profile.add(transmit ? kProfileTxRows : kProfileRxRows);)
         const bool go_on = transmit ? tx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, deadline, counters PCIE_EP_PROFILE(, profile, sampled))
                                     : rx_row<kFp8, kVector>(state, q, scratch, lane, ticket_index, counters, deadline, gate_open, prefixes_known PCIE_EP_PROFILE(, profile, sampled));

@@ -28,7 +28,8 @@ CONTROL = COMMON + ("first_ticket_ns", "last_ticket_ns", "workers_done_ns", "dra
                     "poll_sum", "health_scans", "health_sum", "counts_known_ns", "spare", "prefix_enter_ns",
                     "prefix_counts_ready_ns", "prefix_mailbox_ns", "prefix_published_ns")
 WORKER = COMMON + ("first_claim_ns", "last_row_ns", "tx_rows", "rx_rows", "sampled_tx_rows", "sampled_rx_rows", "ticket_wait_sum",
-                   "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum", "gate_open_ns")
+                   "idle_sum", "tx_flow_wait_sum", "tx_copy_sum", "rx_request_sum", "rx_prefix_wait_sum", "rx_scatter_sum", "gate_open_ns",
+                   "first_look_ns", "first_tagged_ns", "first_entry_ns", "first_request_ns", "first_data_ns")
 PROLOGUE = COMMON + ("layout_ns", "totals_ns", "verdict_ns", "mailbox_free_ns", "mailbox_acked_ns", "counts_ready_ns",
                      "begun_ns", "routes_ns", "masks_ns", "chunk_totals_ns", "plan_ready_ns")
 
@@ -85,8 +86,15 @@ def timeline(records: Dict[str, np.ndarray]) -> Dict[str, float]:
         count = int(np.sum(count))
         return float("nan") if count == 0 else float(np.sum(total)) / count / 1e3
 
+    def median(values) -> float:
+        values = np.asarray(values).reshape(-1)
+        values = values[values > 0]
+        return float("nan") if values.size == 0 else (float(np.median(values)) - zero) / 1e3
+
     out = {f"prologue.{name[:-3]}": first(_col(pro, PROLOGUE, name)) for name in PROLOGUE[4:] + ("exit_ns",)}
     active = wrk[_col(wrk, WORKER, "items") > 0]
+    # Wavefronts whose first row was a received one, claimed before any row had come in.
+    receivers = wrk[(_col(wrk, WORKER, "first_entry_ns") > 0) & (_col(wrk, WORKER, "first_entry_ns") <= _col(wrk, WORKER, "first_request_ns"))]
     out.update({
         "transport.first_role_enter": first(np.concatenate([_col(txc, CONTROL, "enter_ns"), _col(rxc, CONTROL, "enter_ns"), _col(wrk, WORKER, "enter_ns")])),
         "prefix.enter": first(_col(rxc, CONTROL, "prefix_enter_ns")), "prefix.counts_ready_seen": first(_col(rxc, CONTROL, "prefix_counts_ready_ns")),
@@ -100,6 +108,10 @@ def timeline(records: Dict[str, np.ndarray]) -> Dict[str, float]:
         "tx.rows_published_last": last(_col(txc, CONTROL, "workers_done_ns")), "tx.drained_last": last(_col(txc, CONTROL, "drained_ns")),
         "tx.finished_last": last(_col(txc, CONTROL, "finished_ns")), "tx.drain_poll_us": per(_col(txc, CONTROL, "poll_sum"), _col(txc, CONTROL, "polls")),
         "tx.drain_polls": float(np.sum(_col(txc, CONTROL, "polls"))), "tx.drain_misses": float(np.sum(_col(txc, CONTROL, "poll_misses"))),
+        # The way of a payload wavefront's first row (median over the wavefronts whose first row was a received one).
+        **{f"first_row.{name}": median(_col(receivers, WORKER, field)) for name, field in (
+            ("look", "first_look_ns"), ("claim", "first_claim_ns"), ("tag_seen", "first_tagged_ns"), ("entry_read", "first_entry_ns"),
+            ("gate_passed", "gate_open_ns"), ("requested", "first_request_ns"), ("metadata_back", "first_data_ns"))},
         "workers.first_claim": first(_col(wrk, WORKER, "first_claim_ns")), "workers.last_row_end": last(_col(wrk, WORKER, "last_row_ns")),
         "workers.active": float(active.shape[0]),
         "workers.ticket_wait_us": per(_col(wrk, WORKER, "ticket_wait_sum"), _col(wrk, WORKER, "items")),
