@@ -323,7 +323,9 @@ int pcie_ep_get_kernel_times(pcie_ep_runtime* runtime, float* milliseconds3);
  * (csrc/kernels/host_staged/advanced_common.cuh:126-181; docs/pcie-ep/
  * profiling-instrumentation.md): one record of `fields` (32) int64 per role wavefront,
  * rows ordered TX control [0, C), RX control [C, 2C), payload wavefronts
- * [2C, 2C + W), prologue leader [2C + W]; the field meanings are the ProfileField /
+ * [2C, 2C + W), prologue leader [2C + W], epoch begin [2C + W + 1], producer of the
+ * receive prefixes [2C + W + 2] (the last two where they are roles of their own, else
+ * zero); the field meanings are the ProfileField /
  * PrologueProfileField enums of csrc/device_common.h, mirrored in pcie_ep/profiling.py.
  * pcie_ep_profile_read synchronises the device (a diagnostic wait outside the dispatch
  * path, like the reference's handle.profiling.cpu()). */

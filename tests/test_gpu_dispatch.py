@@ -164,6 +164,19 @@ def test_many_experts_narrow_chunks():
         check_case(buffer, "e4096-unique", [333] * 16, expand=False, seed=21)
 
 
+def test_separate_expand_with_more_padding_work_than_rows():
+    """Many local experts and a pool of a few rows: the stand-alone expand's grid is
+    then sized by the alignment gaps it zeroes, not by the rows, and the workgroups
+    beyond the pool must not touch it (128 local experts, a pool of 10 rows)."""
+    with make_buffer(world=2, tmax=5, hidden=256, topk=4, experts=256, channels=3, payload_slots=4, descriptor_slots=4,
+                     fuse_receive_expand=False, receive_expand_mode="scalar") as buffer:
+        check_case(buffer, "wide-grid", [5, 3], alignment=16)
+        check_case(buffer, "wide-grid-empty", [0, 0], alignment=2, seed=9)
+    with make_buffer(world=1, tmax=1, hidden=2048, topk=1, experts=64, channels=2, fuse_receive_expand=False,
+                     receive_expand_mode="scalar") as buffer:
+        check_case(buffer, "wide-grid-one-row", [1], alignment=256, capture=False)
+
+
 def test_numa_bound_staging_segments():
     """The pinned segments can be bound to a NUMA node (the far-node staging of the
     cached-replay configuration); node 0 exists on every box.  Results do not change."""
