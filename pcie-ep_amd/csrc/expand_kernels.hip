@@ -89,19 +89,16 @@ __global__ void __launch_bounds__(kPieceThreads) expand_pieces_kernel(DeviceStat
     const uint32_t row_bytes = uint32_t(hidden) * 2u;
     const int entries = local + 1 + z.dims.num_ranks * local;
     const bool tabled = entries <= kPieceTableEntries;
-    // Row `group` exists in the pool whether or not it is in use (the grid may be wider
-    // than the pool where it is sized by the padding work: those workgroups load nothing):
-    // its loads are issued before anything is known, beside the loads of the count and the tables.
+    // Row `group` exists in the pool whether or not it is in use: its loads are issued
+    // before anything is known, beside the loads of the count and the tables.  (The grid
+    // may be wider than the pool where it is sized by the padding work: a workgroup
+    // beyond the pool loads row 0 instead and never uses it.)
     int64_t row = group;
-    const bool pooled = row < unique_capacity(z.dims);
-    u32x4 value = {0u, 0u, 0u, 0u};
-    int source = 0, expert = -1, ordinal = 0;
-    if (pooled) {
-        value = stream_load_b128(device_resource(state.unique_payload + size_t(row) * hidden, row_bytes), at);
-        source = int(state.unique_source_meta[row * 3]);
-        expert = lane < topk ? int(state.unique_topk_idx[row * topk + lane]) : -1;
-        ordinal = lane < topk ? state.unique_expert_ordinals[row * topk + lane] : 0;
-    }
+    const int64_t first = row < unique_capacity(z.dims) ? row : 0;
+    u32x4 value = stream_load_b128(device_resource(state.unique_payload + size_t(first) * hidden, row_bytes), at);
+    int source = int(state.unique_source_meta[first * 3]);
+    int expert = lane < topk ? int(state.unique_topk_idx[first * topk + lane]) : -1;
+    int ordinal = lane < topk ? state.unique_expert_ordinals[first * topk + lane] : 0;
     // Never beyond the pool, whatever count the sources announced.
     const int64_t announced = *state.unique_count, unique = announced < unique_capacity(z.dims) ? announced : unique_capacity(z.dims);
     const bool failed = load_error_code(state) != 0;
