@@ -174,7 +174,22 @@ __device__ __forceinline__ int wait_ticket(const DeviceState& state, TransportQu
 // elected by a device-scope CAS; it waits for every source's counts_ready,
 // folds the mailboxes in rank order and publishes a generation-valued READY.
 // ---------------------------------------------------------------------------------------
-__device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
+// The producer's first look at every source's counts_ready (lane r: rank r), issued by the
+// kernel's entry code before the role is let in; see RxFirstPoll.
+struct PrefixFirstLook {
+    uint64_t word;
+    bool issued;
+};
+__device__ __forceinline__ PrefixFirstLook prefix_first_look(const DeviceState& state, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks;
+    PrefixFirstLook look{0, true};
+    if (lane < ranks && !(state.fused != 0 && lane == state.local_rank))
+        look.word = host_load_global(signal_at(state.seg[lane], z.counts_ready_offset));
+    return look;
+}
+
+__device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& state, int lane, PrefixFirstLook entry_look PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, local = z.local_experts, channels = z.dims.channels;
     const int me = state.local_rank;
@@ -207,8 +222,9 @@ __device__ __forceinline__ bool compute_receive_prefixes(const DeviceState& stat
     const bool own_from_plan = state.fused != 0;
     // The first look at every source's counts_ready is requested now; its value is
     // used after the address arithmetic below, which so runs inside its round trip.
-    uint64_t first_look = 0;
-    if (lane < ranks && !(own_from_plan && lane == me)) first_look = host_load_global(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
+    uint64_t first_look = entry_look.word;
+    if (!entry_look.issued && lane < ranks && !(own_from_plan && lane == me))
+        first_look = host_load_global(signal_at(const_cast<char*>(lane_segment), z.counts_ready_offset));
     const auto segment_of = [&](int rank) {
         const uint64_t bits = reinterpret_cast<uint64_t>(lane_segment);
         return reinterpret_cast<char*>(uint64_t(uint32_t(__shfl(int(uint32_t(bits)), rank))) | uint64_t(uint32_t(__shfl(int(uint32_t(bits >> 32)), rank))) << 32);
@@ -348,7 +364,7 @@ __device__ __forceinline__ void acknowledge_counts(const DeviceState& state, int
         host_field_store(signal_at(state.seg[lane], z.counts_consumed_offset, state.local_rank), dispatch_epoch(state));
 }
 
-__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile));
+__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane, PrefixFirstLook entry_look PCIE_EP_PROFILE(, RoleProfile& profile));
 
 // One wavefront of the grid (the first RX control to get there) computes the
 // receive prefixes; nobody waits here.
@@ -360,7 +376,7 @@ __device__ __forceinline__ void elect_receive_prefixes(const DeviceState& state,
         claimed = atomicCAS(reinterpret_cast<unsigned long long*>(state.receive_prefix_state), expected, epoch) == 0ull;
     }
     if (!broadcast_first(claimed)) return;
-    produce_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+    produce_receive_prefixes(state, lane, PrefixFirstLook{0, false} PCIE_EP_PROFILE(, profile));
 }
 
 // With payload workgroups of their own, the control workgroups have wavefronts to
@@ -370,16 +386,16 @@ __device__ __forceinline__ void elect_receive_prefixes(const DeviceState& state,
 // elected RX control starts to receive a prefix computation late.
 __device__ __forceinline__ bool dedicated_prefix_producer(const DeviceState& state) { return state.worker_groups > 0 && state.tx_waves + state.rx_waves >= 3; }
 
-__device__ __forceinline__ void receive_prefix_role(const DeviceState& state, int lane) {
+__device__ __forceinline__ void receive_prefix_role(const DeviceState& state, int lane, PrefixFirstLook entry_look) {
     PCIE_EP_PROFILE(RoleProfile profile(state.clock_khz);)
     if (lane == 0) device_store(state.receive_prefix_state, dispatch_epoch(state));
-    produce_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+    produce_receive_prefixes(state, lane, entry_look PCIE_EP_PROFILE(, profile));
     PCIE_EP_PROFILE(profile.save(state.profiling, profile_rows(state.z.dims.channels, state.worker_groups * (state.tx_waves + state.rx_waves)) - 1, lane);)
 }
 
-__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane PCIE_EP_PROFILE(, RoleProfile& profile)) {
+__device__ __forceinline__ void produce_receive_prefixes(const DeviceState& state, int lane, PrefixFirstLook entry_look PCIE_EP_PROFILE(, RoleProfile& profile)) {
     const uint64_t epoch = dispatch_epoch(state);
-    const bool success = compute_receive_prefixes(state, lane PCIE_EP_PROFILE(, profile));
+    const bool success = compute_receive_prefixes(state, lane, entry_look PCIE_EP_PROFILE(, profile));
     // The results were written through; they are complete once this wavefront's
     // stores have been acknowledged.  Local consumers come first, the ACK to the
     // sources (which nobody on this GPU waits for) second.
@@ -601,7 +617,32 @@ __device__ __forceinline__ void tx_control(const DeviceState& state, TransportQu
 // ---------------------------------------------------------------------------------------
 // RX control
 // ---------------------------------------------------------------------------------------
-__device__ __forceinline__ void rx_control(const DeviceState& state, TransportQueues& q, int channel, int lane) {
+// The first look of a receive control at its descriptor queues (entry `ahead` of every
+// source's queue): the same load as in the first pass of rx_control's loop, issued by
+// the kernel's entry code while the role still waits to be let in (the queues it hands
+// tickets out through are being reset), so that the round trip over the host link and
+// that wait overlap.
+struct RxFirstPoll {
+    u32x4 published;
+    bool issued;
+};
+__device__ __forceinline__ RxFirstPoll rx_first_poll(const DeviceState& state, int channel, int lane) {
+    const SegmentLayout& z = state.z;
+    const int ranks = z.dims.num_ranks, me = state.local_rank;
+    const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
+    const int source = lane / lookahead, ahead = lane % lookahead;
+    const bool member = source < ranks && source != me;
+    const bool replica = member && reads_replica(z.dims, source, me);
+    const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
+    char* segment = state.seg[member ? source : me];
+    Descriptor* descriptor = replica ? replica_descriptor_at(z, segment, channel, my_domain, me, member ? ahead : 0)
+                                     : descriptor_at(z, segment, channel, me, member ? ahead : 0);
+    RxFirstPoll poll{{0u, 0u, 0u, 0u}, true};
+    if (member) poll.published = host_load_b128_at(descriptor);
+    return poll;
+}
+
+__device__ __forceinline__ void rx_control(const DeviceState& state, TransportQueues& q, int channel, int lane, RxFirstPoll first_poll) {
     const SegmentLayout& z = state.z;
     const int ranks = z.dims.num_ranks, me = state.local_rank;
     const uint64_t begin = now_ticks();
@@ -629,8 +670,12 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
     int64_t not_ready = 0, ring_waits = 0;
     bool failed = false;
     while (!failed && !prefix_failed) {
-        if (broadcast_first(aborted(q) ? 1 : 0)) break;
-        if (!counts_known) {
+        // The pass that consumes the look taken at entry goes straight to it: the abort word and the
+        // prefixes' state (two trips to device memory) cannot have anything to say a few microseconds
+        // into the launch, and are looked at from the second pass on.
+        const bool entry_pass = first_poll.issued && consumed == 0 && issued == 0 && !counts_known;
+        if (!entry_pass && broadcast_first(aborted(q) ? 1 : 0)) break;
+        if (!counts_known && !entry_pass) {
             const int verdict = receive_prefix_verdict(state, epoch, lane);
             if (verdict < 0) {
                 prefix_failed = true;
@@ -655,7 +700,13 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
         // One 16-byte load brings READY together with the slot and token it guards.
         u32x4 published = {0u, 0u, 0u, 0u};
         PCIE_EP_PROFILE(const uint64_t poll_begin = profile.now(); profile.add(kProfilePolls);)
-        if (want) published = host_load_b128_at(descriptor);
+        if (entry_pass) {
+            // Nothing has been consumed and the counts are not known: this pass would load exactly what was loaded at entry.
+            published = first_poll.published;
+            first_poll.issued = false;
+        } else if (want) {
+            published = host_load_b128_at(descriptor);
+        }
         PCIE_EP_PROFILE(profile.add(kProfilePollSum, profile.now() - poll_begin);)
         const bool ready = want && (uint64_t(published[0]) | uint64_t(published[1]) << 32) == sequence(epoch, ordinal);
         const uint64_t ready_lanes = __ballot(ready);
@@ -1432,11 +1483,27 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
             return;
         }
         block -= prologue_groups;
+    }
+    const int channel_groups = control_groups(state);
+    // Which control this wavefront is, if any - known before the role may start.  The two roles whose first
+    // action is a read over the host link issue it now: a receive control its first look at the descriptor
+    // queues, the producer of the prefixes its first look at the sources' counts_ready.  The wait for the epoch
+    // begin (the queues are being reset; 3 us into the launch) then runs inside that round trip (4.4 us).
+    const bool control_of_pair = payload_groups && block < channel_groups;
+    const bool transmit_group = control_of_pair && (block + prologue_groups) % kControlXcds == 0;
+    const bool prefix_producer = transmit_group && block / 2 == 0 && wave == 2 && dedicated_prefix_producer(state);
+    int receive_channel = -1;
+    if (control_of_pair && !transmit_group && wave < 2 && 2 * (block / 2) + wave < channels) receive_channel = 2 * (block / 2) + wave;
+    if (!payload_groups && block < channel_groups && wave == 1) receive_channel = block;
+    RxFirstPoll first_poll{{0u, 0u, 0u, 0u}, false};
+    if (receive_channel >= 0) first_poll = rx_first_poll(state, receive_channel, lane);
+    PrefixFirstLook first_look{0, false};
+    if (prefix_producer) first_look = prefix_first_look(state, lane);
+    if (state.fused) {
         begun = __syncthreads_or(threadIdx.x == 0 ? int(wait_for_begin(state, q)) : 0) != 0;
     } else if (__syncthreads_or(threadIdx.x == 0 ? int(load_error_code(state) != 0) : 0)) {
         return;  // the prologue kernel in front of this one failed
     }
-    const int channel_groups = control_groups(state);
     if (block >= channel_groups + payload_groups) {
         if (begun) local_rows<kVector>(state, q, lane);
         return finish_role(state, q, lane, roles);
@@ -1457,19 +1524,19 @@ __global__ void __launch_bounds__(kTransportMaxThreads) transport_kernel(DeviceS
                 if (channel >= channels) return;
                 if (begun) {
                     if (transmit) tx_control(state, q, channel, lane);
-                    else rx_control(state, q, channel, lane);
+                    else rx_control(state, q, channel, lane, first_poll);
                 }
                 return finish_role(state, q, lane, roles);
             }
             // The producer of the receive prefixes: third wavefront of the first transmit control workgroup.
-            if (pair != 0 || !transmit || wave != 2 || !dedicated_prefix_producer(state)) return;
-            if (begun) receive_prefix_role(state, lane);
+            if (!prefix_producer) return;
+            if (begun) receive_prefix_role(state, lane, first_look);
             return finish_role(state, q, lane, roles);
         }
         if (wave < 2) {
             if (begun) {
                 if (wave == 0) tx_control(state, q, block, lane);
-                else rx_control(state, q, block, lane);
+                else rx_control(state, q, block, lane, first_poll);
             }
             return finish_role(state, q, lane, roles);
         }
