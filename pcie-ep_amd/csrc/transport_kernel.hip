@@ -626,19 +626,34 @@ struct RxFirstPoll {
     u32x4 published;
     bool issued;
 };
+// Which descriptor queue a lane of a receive control looks at: up to 64 / P entries ahead in every source's queue.
+struct RxLane {
+    int lookahead, source, ahead, my_domain;
+    bool member, replica;
+    __device__ __forceinline__ RxLane(const DeviceState& state, int lane) {
+        const SegmentLayout& z = state.z;
+        const int ranks = z.dims.num_ranks, me = state.local_rank;
+        lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
+        source = lane / lookahead;
+        ahead = lane % lookahead;
+        member = source < ranks && source != me;
+        // A source of another domain is read from the replica ring its relay fills
+        // for this rank's domain (advanced_common.cuh:237-247).
+        replica = member && reads_replica(z.dims, source, me);
+        my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
+    }
+    // Entry `ordinal` of the lane's queue (entry 0 of the own queue for a lane without one: never loaded).
+    __device__ __forceinline__ Descriptor* entry(const DeviceState& state, int channel, int ordinal) const {
+        const SegmentLayout& z = state.z;
+        const int me = state.local_rank;
+        char* segment = state.seg[member ? source : me];
+        return replica ? replica_descriptor_at(z, segment, channel, my_domain, me, ordinal) : descriptor_at(z, segment, channel, me, ordinal);
+    }
+};
 __device__ __forceinline__ RxFirstPoll rx_first_poll(const DeviceState& state, int channel, int lane) {
-    const SegmentLayout& z = state.z;
-    const int ranks = z.dims.num_ranks, me = state.local_rank;
-    const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
-    const int source = lane / lookahead, ahead = lane % lookahead;
-    const bool member = source < ranks && source != me;
-    const bool replica = member && reads_replica(z.dims, source, me);
-    const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
-    char* segment = state.seg[member ? source : me];
-    Descriptor* descriptor = replica ? replica_descriptor_at(z, segment, channel, my_domain, me, member ? ahead : 0)
-                                     : descriptor_at(z, segment, channel, me, member ? ahead : 0);
+    const RxLane at(state, lane);
     RxFirstPoll poll{{0u, 0u, 0u, 0u}, true};
-    if (member) poll.published = host_load_b128_at(descriptor);
+    if (at.member) poll.published = host_load_b128_at(at.entry(state, channel, at.ahead));
     return poll;
 }
 
@@ -655,11 +670,9 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
     // (how many rows each source sends on this channel) are only needed to know
     // when to stop; the payload wavefronts wait for the prefixes after they have
     // requested a row, before they compute where it goes.
-    const int lookahead = kWave / ranks > 32 ? 32 : kWave / ranks;
-    const int source = lane / lookahead, ahead = lane % lookahead;
-    const bool member = source < ranks && source != me;
-    const bool replica = member && reads_replica(z.dims, source, me);
-    const int my_domain = z.dims.domains ? z.dims.rank_domain[me] : 0;
+    const RxLane at(state, lane);
+    const int lookahead = at.lookahead, source = at.source, ahead = at.ahead, my_domain = at.my_domain;
+    const bool member = at.member, replica = at.replica;
     int expected = member ? 0x7FFFFFFF : 0, total = 0x7FFFFFFF;
     bool counts_known = false, prefix_failed = false;
     const uint64_t below = lanes_below(lane);
@@ -692,11 +705,7 @@ __device__ __forceinline__ void rx_control(const DeviceState& state, TransportQu
         if (counts_known && issued >= total) break;
         const int ordinal = consumed + ahead;
         const bool want = member && ordinal < expected;
-        // A source of another domain is read from the replica ring its relay fills
-        // for this rank's domain (advanced_common.cuh:237-247).
-        char* segment = state.seg[member ? source : me];
-        Descriptor* descriptor = replica ? replica_descriptor_at(z, segment, channel, my_domain, me, want ? ordinal : 0)
-                                         : descriptor_at(z, segment, channel, me, want ? ordinal : 0);
+        Descriptor* descriptor = at.entry(state, channel, want ? ordinal : 0);
         // One 16-byte load brings READY together with the slot and token it guards.
         u32x4 published = {0u, 0u, 0u, 0u};
         PCIE_EP_PROFILE(const uint64_t poll_begin = profile.now(); profile.add(kProfilePolls);)
