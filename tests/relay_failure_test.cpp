@@ -140,7 +140,9 @@ int happy_path_pinned() {
     if (outgoing->token_index != 5) return fail("replica descriptor names another token");
     const char* copy = replica_slot_at(w.z, w.replica[kFar], 0, outgoing->payload_slot);
     if (static_cast<unsigned char>(copy[0]) != 0x45 || static_cast<unsigned char>(copy[w.z.payload_bytes - 1]) != 0x45) return fail("replica payload differs");
-    if (acquire(ack_at(w.z, w.own(), 0, 1, kRanks + kFar)) != sequence(1, 5)) return fail("the source slot was not ACKed on behalf of the relay endpoint");
+    // The relay publishes the replica descriptor first and ACKs the source slot right after.
+    if (!eventually([&] { return acquire(ack_at(w.z, w.own(), 0, 1, kRanks + kFar)) == sequence(1, 5); }))
+        return fail("the source slot was not ACKed on behalf of the relay endpoint");
     // Rank 1 consumes the replica row.
     release(replica_ack_at(w.z, w.own(), 0, kFar, outgoing->payload_slot, 1), sequence(1, 5));
     release(replica_credit_at(w.z, w.own(), 0, kFar, 1), sequence(1, 0));
@@ -153,11 +155,20 @@ int happy_path_pinned() {
     return 0;
 }
 
-int expect_code(const char* name, uint64_t code, int timeout_ms, void (*drive)(World&)) {
+// True once every flow of the relay has taken up `epoch`.
+bool flows_entered(const NumaRelay& relay, uint64_t epoch) {
+    std::vector<RelayFlowRecord> records(8);
+    const int flows = relay.diagnostics(records.data(), int(records.size()));
+    for (int i = 0; i < flows; ++i)
+        if (records[i].epoch != epoch) return false;
+    return flows > 0;
+}
+
+int expect_code(const char* name, uint64_t code, int timeout_ms, void (*drive)(World&, const NumaRelay&)) {
     World w;
     {
         NumaRelay relay(w.z, 0, w.segments, w.replica, options(timeout_ms));
-        drive(w);
+        drive(w, relay);
         if (!eventually([&] { return w.failed() != 0; })) return fail(std::string(name) + ": no failure code was stored");
         if (w.failed() != code) return fail(std::string(name) + ": code " + std::to_string(w.failed()) + ", expected " + std::to_string(code));
         // Nothing was copied or announced for the failed row.
@@ -203,21 +214,23 @@ int worker_exception() {
 int main() {
     int status = happy_path_pinned();
     if (!status) std::printf("happy path with pinned workers ok\n");
-    if (!status) status = expect_code("epoch changed before the drain", 101, 20000, [](World& w) {
+    if (!status) status = expect_code("epoch changed before the drain", 101, 20000, [](World& w, const NumaRelay& relay) {
         w.begin_epoch(1, 1);  // one row expected, none published
-        std::this_thread::sleep_for(std::chrono::milliseconds(20));
+        // The next epoch begins once the flows are inside this one (a flow that first looks after the second
+        // announcement would simply start there).
+        eventually([&] { return flows_entered(relay, 1); });
         w.begin_epoch_early(2);
     });
-    if (!status) status = expect_code("no progress", 102, 60, [](World& w) { w.begin_epoch(1, 1); });
-    if (!status) status = expect_code("slot outside the ring", 103, 20000, [](World& w) {
+    if (!status) status = expect_code("no progress", 102, 60, [](World& w, const NumaRelay&) { w.begin_epoch(1, 1); });
+    if (!status) status = expect_code("slot outside the ring", 103, 20000, [](World& w, const NumaRelay&) {
         w.begin_epoch(1, 1);
         w.publish(1, 0, kSlots, 2, 2, 1u << 1);
     });
-    if (!status) status = expect_code("identity mismatch", 104, 20000, [](World& w) {
+    if (!status) status = expect_code("identity mismatch", 104, 20000, [](World& w, const NumaRelay&) {
         w.begin_epoch(1, 1);
         w.publish(1, 0, 0, 2, 6, 1u << 1);
     });
-    if (!status) status = expect_code("no destination in the domain", 105, 20000, [](World& w) {
+    if (!status) status = expect_code("no destination in the domain", 105, 20000, [](World& w, const NumaRelay&) {
         w.begin_epoch(1, 1);
         w.publish(1, 0, 0, 2, 2, 1u << 0);
     });

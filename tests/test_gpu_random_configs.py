@@ -4,13 +4,16 @@ rank, top-k, row length (vector and scalar paths, multi-pass rows), channels,
 ring sizes down to one slot, ragged and empty token counts, both layouts, both
 wires, alignments up to 256, missing weights, route patterns, wavefront counts
 and fused / separate expansion.  Two dispatches per buffer, so slot, descriptor
-and plan reuse across epochs is covered too."""
+and plan reuse across epochs is covered too.  A second walk takes the same
+configurations through cached layouts, static and dynamic graph replays and the
+prologue as a launch of its own."""
 
 from __future__ import annotations
 
 import random
 
 import pytest
+import torch
 
 from helpers import make_inputs, run_dispatch, verify_captured, verify_dispatch
 
@@ -103,3 +106,72 @@ def test_random_configurations_through_the_relay(first):
                 verify_captured(buffer.peers, inputs, c["rank"], c["world"], c["experts"], c["topk"], fp8_wire=c["fp8"],
                                 with_weights=c["weights"])
                 del result
+
+
+@pytest.mark.parametrize("first", range(2000, 2060, 20))
+def test_random_configurations_through_cached_layouts_and_graphs(first):
+    """Every configuration: one eager dispatch, then three replays of a cached
+    layout, of a static cached graph or of a dynamic graph (drawn per case) with
+    fresh payload and weights on every rank, fresh routes on the other ranks and -
+    where the graph recomputes them - on the own rank, and an eager dispatch between
+    the replays; three cases in ten run the prologue as a launch of its own."""
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    for case in range(first, first + 20):
+        c = draw(case)
+        rng = random.Random(case * 13 + 5)
+        split = rng.random() < 0.3
+        mode = rng.choice(["dynamic", "static", "cached"])
+        print(f"case {case}: {c} split_launch={split} mode={mode}", flush=True)
+        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
+                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
+                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar", enable_graph=True)
+        me, expand, weighted = c["rank"], c["expand"], c["weights"]
+
+        def check(result, inputs):
+            verify_dispatch(result, inputs, me, c["world"], c["experts"], c["topk"], expand, c["alignment"], expand, with_weights=weighted,
+                            fp8_wire=c["fp8"])
+
+        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
+                                config=config, num_ranks=c["world"], rank=me, tx_waves=c["waves"][0], rx_waves=c["waves"][1],
+                                worker_groups=c["waves"][2], split_launch=split) as buffer:
+            inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10,
+                                 gaussian=c["fp8"], heavy_tail=c["fp8"])
+            result, (x, idx, weights) = run_dispatch(buffer, inputs, expand=expand, alignment=c["alignment"], zero_padding=expand,
+                                                     with_weights=weighted)
+            check(result, inputs)
+            own_weights = weights if weighted else None
+            cache = buffer.cache_layout(result[3]) if mode != "dynamic" else None
+            del result
+            graph = None
+            if mode == "dynamic":
+                graph = buffer.capture_dispatch(x, idx, own_weights, do_expand=expand, expert_alignment=c["alignment"], do_zero_padding=expand)
+            elif mode == "static":
+                graph = buffer.capture_dispatch(x, topk_weights=own_weights, handle=cache, do_expand=expand, do_zero_padding=expand)
+            for step in range(3):
+                fresh = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + 1 + step,
+                                    gaussian=c["fp8"], heavy_tail=c["fp8"])
+                x.copy_(fresh[me][0])
+                weights.copy_(fresh[me][2])
+                if mode == "dynamic":
+                    idx.copy_(fresh[me][1])
+                inputs = list(fresh)
+                inputs[me] = (x.cpu(), idx.cpu(), weights.cpu())
+                if buffer.peers is not None:
+                    for source, (peer_x, peer_idx, peer_weights) in enumerate(inputs):
+                        if source != me:
+                            buffer.peers.set_source(source, peer_x, peer_idx, peer_weights if weighted else None)
+                    buffer.peers.start(1)
+                if graph is not None:
+                    result = graph.replay()
+                else:
+                    result = buffer.dispatch(x, topk_weights=own_weights, handle=cache, do_expand=expand, do_zero_padding=expand)
+                torch.cuda.synchronize()
+                if buffer.peers is not None:
+                    buffer.peers.wait(30_000)
+                check(result, inputs)
+                del result
+                if step == 1:
+                    result, _ = run_dispatch(buffer, inputs, expand=expand, alignment=c["alignment"], zero_padding=expand, with_weights=weighted)
+                    check(result, inputs)
+                    del result
