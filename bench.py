@@ -27,6 +27,7 @@ dispatch checked bit for bit against the oracle.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -247,6 +248,11 @@ def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, ver
         buffer.peers.wait_staged(120_000)
         # The emulator on its own: the first epoch is staged while the GPU is idle.
         stage_seconds = time.perf_counter() - stage_started
+        # The interpreter's cyclic collector stays out of the measured passes, as under
+        # `timeit`: a full collection of this process's heap takes 40 ms, some 700
+        # small dispatches, and would land inside one of them.
+        gc.collect()
+        gc.disable()
         for _ in range(warmup):
             result = buffer.dispatch(x, idx, weights, do_expand=True, async_with_compute_stream=True)
             del result
@@ -319,6 +325,7 @@ def run_workload(inputs, tokens, topk, wire, channels, steps, warmup, peaks, ver
             unique, expanded = int(probe.unique_count.cpu()), int(probe.expanded_count.cpu())
         del result
     finally:
+        gc.enable()
         buffer.close()
 
     mean = lambda values: sum(values) / len(values)
@@ -386,14 +393,19 @@ def graph_replay_sweep(topk, channels, sizes=(16, 128, 512, 2048, 8192), replays
             cache = buffer.cache_layout(result[3])
             del result
             graph = buffer.capture_dispatch(x, topk_weights=weights, handle=cache, do_expand=True)
-            for _ in range(3):
-                graph.replay(async_with_compute_stream=True)
-            torch.cuda.synchronize()
-            started = time.perf_counter()
-            for _ in range(replays):
-                graph.replay(async_with_compute_stream=True)
-            torch.cuda.synchronize()
-            replay_us = (time.perf_counter() - started) / replays * 1e6
+            gc.collect()
+            gc.disable()  # as in run_workload
+            try:
+                for _ in range(3):
+                    graph.replay(async_with_compute_stream=True)
+                torch.cuda.synchronize()
+                started = time.perf_counter()
+                for _ in range(replays):
+                    graph.replay(async_with_compute_stream=True)
+                torch.cuda.synchronize()
+                replay_us = (time.perf_counter() - started) / replays * 1e6
+            finally:
+                gc.enable()
             result = graph.replay()
             torch.cuda.synchronize()
             buffer.peers.wait(120_000)
