@@ -105,3 +105,36 @@ def test_four_runtimes_with_the_prologue_as_a_launch_of_its_own():
     dispatch and once with the prologue kernel in front."""
     for split in (False, True):
         run_world(4, [33, 64, 0, 17], 512, 4, 32, ROUNDS[:3], channels=2, payload_slots=3, descriptor_slots=2, worker_groups=4, split_launch=split)
+
+
+def test_random_worlds_of_runtimes():
+    """A seeded walk over worlds of two to four runtimes: world size, ragged and
+    empty token counts, row lengths (vector and scalar paths), top-k, experts per
+    rank, channels, ring sizes down to one slot, payload workgroups, both wires,
+    both launch shapes, and two to four rounds of random patterns and layouts each."""
+    import random
+
+    for case in range(60):
+        rng = random.Random(case * 31 + 7)
+        world = rng.choice([2, 2, 3, 4])
+        local = rng.choice([1, 2, 4, 8, 16])
+        experts = world * local
+        topk = rng.randint(1, min(8, experts))
+        hidden = rng.choice([8, 64, 129, 512, 1024, 2048, 7168])
+        tmax = rng.choice([1, 5, 33, 64, 96, 200])
+        tokens = [rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)]
+        if max(tokens) == 0:
+            tokens[0] = 1
+        fp8 = rng.random() < 0.3
+        config = dict(channels=rng.randint(1, 4), payload_slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptor_slots=rng.choice([1, 2, 3, 5, 16, 256]),
+                      worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3)
+        if fp8:
+            config.update(stage=7, wire_dtype="fp8_e4m3")
+        rounds = []
+        for _ in range(rng.randint(2, 4)):
+            pattern = rng.choice(["random", "random", "multicast", "hotspot", "local", "none", "partial"])
+            if pattern in ("hotspot", "local") and topk > local:
+                pattern = "random"
+            expand = rng.random() < 0.7
+            rounds.append((pattern, expand, rng.choice([1, 2, 8, 16, 128]) if expand else 1, rng.random() < 0.8))
+        run_world(world, tokens, hidden, topk, experts, rounds, **config)
