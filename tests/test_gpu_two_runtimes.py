@@ -28,7 +28,7 @@ def make_world(world, tmax, hidden, topk, experts, shared, **config):
     from pcie_ep import HostStagedConfig, HostStagedEPBuffer
 
     config.setdefault("timeout_ms", 4000)
-    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "worker_groups", "split_launch") if key in config}
+    extra = {key: config.pop(key) for key in ("tx_waves", "rx_waves", "worker_groups", "split_launch", "rank_numa_nodes") if key in config}
     from pcie_ep.streams import masked_stream
 
     # The ranks' kernels wait for each other and must run at the same time: each rank gets a quarter of the compute
@@ -64,6 +64,7 @@ def run_world(world, tokens, hidden, topk, experts, rounds, **config):
     if CALLER is None:
         CALLER = torch.cuda.Stream()
     shared = SharedSegments()
+    nodes = config.get("rank_numa_nodes")
     buffers = make_world(world, max(tokens), hidden, topk, experts, shared, **config)
     try:
         assert all(buffer.peers is None for buffer in buffers)
@@ -78,7 +79,7 @@ def run_world(world, tokens, hidden, topk, experts, rounds, **config):
                 for rank, result in enumerate(results):
                     # What rank r received is what the OTHER kernels published: this verifies their transmit side too.
                     verify_dispatch(result, inputs, rank, world, experts, topk, expand, alignment, expand, with_weights=weights,
-                                    fp8_wire=config.get("wire_dtype") == "fp8_e4m3")
+                                    fp8_wire=config.get("wire_dtype") == "fp8_e4m3", **({"rank_numa_nodes": nodes} if nodes else {}))
                 del results
     finally:
         for buffer in buffers:
@@ -107,14 +108,19 @@ def test_four_runtimes_with_the_prologue_as_a_launch_of_its_own():
         run_world(4, [33, 64, 0, 17], 512, 4, 32, ROUNDS[:3], channels=2, payload_slots=3, descriptor_slots=2, worker_groups=4, split_launch=split)
 
 
-def test_random_worlds_of_runtimes():
+@pytest.mark.parametrize("relay", [False, True], ids=["direct", "relay"])
+def test_random_worlds_of_runtimes(relay):
     """A seeded walk over worlds of two to four runtimes: world size, ragged and
     empty token counts, row lengths (vector and scalar paths), top-k, experts per
     rank, channels, ring sizes down to one slot, payload workgroups, both wires,
-    both launch shapes, and two to four rounds of random patterns and layouts each."""
+    both launch shapes, and two to four rounds of random patterns and layouts each.
+    In relay mode the ranks are dealt onto two to four NUMA domains and every
+    runtime runs its own relay workers: a row for another domain goes from the
+    publishing kernel through a CPU relay worker and a replica ring to the
+    consuming kernel."""
     import random
 
-    for case in range(60):
+    for case in range(40 if relay else 60):
         rng = random.Random(case * 31 + 7)
         world = rng.choice([2, 2, 3, 4])
         local = rng.choice([1, 2, 4, 8, 16])
@@ -130,6 +136,12 @@ def test_random_worlds_of_runtimes():
                       worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3)
         if fp8:
             config.update(stage=7, wire_dtype="fp8_e4m3")
+        if relay:
+            domains = rng.randint(2, min(4, world))
+            nodes = tuple(rng.randrange(domains) for _ in range(world))
+            if len(set(nodes)) < 2:
+                nodes = tuple(index % 2 for index in range(world))
+            config.update(stage=8, numa_mode="relay", replica_slots=rng.choice([1, 2, 4, 16]), rank_numa_nodes=nodes)
         rounds = []
         for _ in range(rng.randint(2, 4)):
             pattern = rng.choice(["random", "random", "multicast", "hotspot", "local", "none", "partial"])
