@@ -150,3 +150,98 @@ def test_random_worlds_of_runtimes(relay):
             expand = rng.random() < 0.7
             rounds.append((pattern, expand, rng.choice([1, 2, 8, 16, 128]) if expand else 1, rng.random() < 0.8))
         run_world(world, tokens, hidden, topk, experts, rounds, **config)
+
+
+def test_worlds_of_runtimes_replaying_captured_dispatches():
+    """What a serving loop on every rank does: each runtime of a world captures its
+    dispatch into a hipGraph (with a cached layout, or recomputing the routes on
+    every replay) and the ranks replay against each other, three times with fresh
+    payload, weights and - without a cached layout - routes.  Thirty seeded worlds
+    of two to four runtimes, three in ten in relay mode."""
+    import random
+
+    from pcie_ep import SharedSegments
+
+    global CALLER
+    if CALLER is None:
+        CALLER = torch.cuda.Stream()
+    for case in range(30):
+        rng = random.Random(case * 37 + 11)
+        world = rng.choice([2, 2, 3, 4])
+        local = rng.choice([1, 2, 4, 8, 16])
+        experts = world * local
+        topk = rng.randint(1, min(8, experts))
+        hidden = rng.choice([8, 64, 129, 512, 1024, 2048, 7168])
+        tmax = rng.choice([1, 5, 33, 64, 96, 200])
+        tokens = [rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)]
+        if max(tokens) == 0:
+            tokens[0] = 1
+        fp8 = rng.random() < 0.3
+        config = dict(channels=rng.randint(1, 4), payload_slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptor_slots=rng.choice([1, 2, 3, 5, 16, 256]),
+                      worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3, enable_graph=True)
+        if fp8:
+            config.update(stage=7, wire_dtype="fp8_e4m3")
+        nodes = None
+        if rng.random() < 0.3:
+            domains = rng.randint(2, min(4, world))
+            nodes = tuple(rng.randrange(domains) for _ in range(world))
+            if len(set(nodes)) < 2:
+                nodes = tuple(index % 2 for index in range(world))
+            config.update(stage=8, numa_mode="relay", replica_slots=rng.choice([1, 2, 4, 16]), rank_numa_nodes=nodes)
+        expand = rng.random() < 0.7
+        alignment = rng.choice([1, 2, 8, 16, 128]) if expand else 1
+        weighted = rng.random() < 0.8
+        cached = rng.random() < 0.5
+        patterns = [rng.choice(["random", "multicast", "hotspot", "local", "none", "partial"]) for _ in range(3)]
+        patterns = ["random" if pattern in ("hotspot", "local") and topk > local else pattern for pattern in patterns]
+        print(f"case {case}: world={world} tokens={tokens} hidden={hidden} topk={topk} experts={experts} {config} expand={expand} "
+              f"alignment={alignment} weighted={weighted} cached={cached} patterns={patterns}", flush=True)
+        extra = {"rank_numa_nodes": nodes} if nodes else {}
+
+        def check(results, inputs):
+            with torch.cuda.stream(CALLER):
+                for rank, result in enumerate(results):
+                    verify_dispatch(result, inputs, rank, world, experts, topk, expand, alignment, expand, with_weights=weighted, fp8_wire=fp8, **extra)
+
+        shared = SharedSegments()
+        buffers = make_world(world, max(tokens), hidden, topk, experts, shared, **config)
+        try:
+            inputs = make_inputs(world, tokens, hidden, experts, topk, patterns[0], seed=case)
+            resident = [tuple(item.cuda() for item in inputs[rank]) for rank in range(world)]
+            torch.cuda.synchronize()
+            with torch.cuda.stream(CALLER):
+                results = [buffer.dispatch(x, idx, w if weighted else None, do_expand=expand, expert_alignment=alignment, do_zero_padding=expand,
+                                           async_with_compute_stream=True) for buffer, (x, idx, w) in zip(buffers, resident)]
+            torch.cuda.synchronize()
+            check(results, inputs)
+            caches = [buffer.cache_layout(result[3]) if cached else None for buffer, result in zip(buffers, results)]
+            del results
+            torch.cuda.synchronize()
+            graphs = []
+            for buffer, (x, idx, w), cache in zip(buffers, resident, caches):
+                if cached:
+                    graphs.append(buffer.capture_dispatch(x, topk_weights=w if weighted else None, handle=cache, do_expand=expand, do_zero_padding=expand))
+                else:
+                    graphs.append(buffer.capture_dispatch(x, idx, w if weighted else None, do_expand=expand, expert_alignment=alignment,
+                                                          do_zero_padding=expand))
+            for step, pattern in enumerate(patterns):
+                fresh = make_inputs(world, tokens, hidden, experts, topk, patterns[0] if cached else pattern, seed=case * 7 + step + 1)
+                current = []
+                for rank, (x, idx, w) in enumerate(resident):
+                    x.copy_(fresh[rank][0])
+                    w.copy_(fresh[rank][2])
+                    if not cached:
+                        idx.copy_(fresh[rank][1])
+                    current.append((x.cpu(), idx.cpu(), w.cpu()))
+                torch.cuda.synchronize()
+                # Every rank's replay is submitted before any is waited for, as the eager dispatches are.
+                with torch.cuda.stream(CALLER):
+                    results = [graph.replay(async_with_compute_stream=True) for graph in graphs]
+                torch.cuda.synchronize()
+                check(results, current)
+                del results
+                torch.cuda.synchronize()
+        finally:
+            for buffer in buffers:
+                buffer.close()
+            shared.close()
