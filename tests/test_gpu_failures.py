@@ -182,3 +182,61 @@ def test_epoch_exhaustion_is_code_20(inputs):
         print("case: epoch counter set to 2^32 - 1", flush=True)
         buffer.runtime.set_test_epoch(2**32 - 1)
         failing_dispatch(buffer, inputs, 20)
+
+
+def test_random_configurations_with_a_faulty_peer():
+    """Forty configurations of the seeded walk (world size, ring sizes, row lengths,
+    wavefront counts, both wires, both layouts), each with one fault injected into
+    one emulated peer: counts_ready withheld (12), the last payload ACK withheld
+    (15 when this rank sends that peer a row), a wrong payload identity, an
+    out-of-range slot or an out-of-range ordinal (18 when that peer sends this rank
+    a row).  The dispatch ends with exactly that code - or cleanly, where the routes
+    give the fault nothing to act on - well inside the time limit."""
+    import random
+    import time
+
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+    from test_gpu_random_configs import draw
+
+    for case in range(4000, 4040):
+        c = draw(case)
+        if c["world"] == 1:
+            continue
+        rng = random.Random(case * 41 + 3)
+        me, world, experts, topk = c["rank"], c["world"], c["experts"], c["topk"]
+        local = experts // world
+        peer = rng.choice([rank for rank in range(world) if rank != me])
+        fault = rng.choice([FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE, FAULT_SLOT_RANGE, FAULT_RANK_ORDINAL])
+        inputs = make_inputs(world, c["tokens"], c["hidden"], experts, topk, c["pattern"], seed=case * 10, gaussian=c["fp8"], heavy_tail=c["fp8"])
+        peer_sends = bool(((inputs[peer][1] >= me * local) & (inputs[peer][1] < (me + 1) * local)).any())
+        this_rank_sends = bool(((inputs[me][1] >= peer * local) & (inputs[me][1] < (peer + 1) * local)).any())
+        if fault == FAULT_NO_COUNTS_READY:
+            expected = 12
+        elif fault == FAULT_NO_LAST_ACK:
+            expected = 15 if this_rank_sends else 0
+        else:
+            expected = 18 if peer_sends else 0
+        print(f"case {case}: {c} peer={peer} fault={fault} expected code {expected}", flush=True)
+        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=300,
+                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
+                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
+        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=topk, num_experts=experts, config=config,
+                                num_ranks=world, rank=me, tx_waves=c["waves"][0], rx_waves=c["waves"][1], worker_groups=c["waves"][2]) as buffer:
+            buffer.peers.inject_fault(peer, fault)
+            for source, (x, idx, weights) in enumerate(inputs):
+                if source != me:
+                    buffer.peers.set_source(source, x, idx, weights if c["weights"] else None)
+            buffer.peers.start(1)
+            x, idx, weights = (item.cuda() for item in inputs[me])
+            began = time.perf_counter()
+            result = buffer.dispatch(x, idx, weights if c["weights"] else None, do_expand=c["expand"], expert_alignment=c["alignment"],
+                                     do_zero_padding=c["expand"])
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - began
+            if expected:
+                buffer.peers.cancel()
+            else:
+                buffer.peers.wait(30_000)
+            error = result[3].error.cpu().tolist()
+            assert error[0] == expected, f"expected device error {expected}, got {error}"
+            assert elapsed < 3.0, f"the dispatch took {elapsed:.2f} s"
