@@ -195,8 +195,7 @@ def test_random_configurations_with_a_faulty_peer():
     import random
     import time
 
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
-    from test_gpu_random_configs import draw
+    from test_gpu_random_configs import draw, walk_buffer, walk_inputs
 
     for case in range(4000, 4040):
         c = draw(case)
@@ -207,7 +206,7 @@ def test_random_configurations_with_a_faulty_peer():
         local = experts // world
         peer = rng.choice([rank for rank in range(world) if rank != me])
         fault = rng.choice([FAULT_NO_COUNTS_READY, FAULT_NO_LAST_ACK, FAULT_WRONG_SEQUENCE, FAULT_SLOT_RANGE, FAULT_RANK_ORDINAL])
-        inputs = make_inputs(world, c["tokens"], c["hidden"], experts, topk, c["pattern"], seed=case * 10, gaussian=c["fp8"], heavy_tail=c["fp8"])
+        inputs = walk_inputs(c, case * 10)
         peer_sends = bool(((inputs[peer][1] >= me * local) & (inputs[peer][1] < (me + 1) * local)).any())
         this_rank_sends = bool(((inputs[me][1] >= peer * local) & (inputs[me][1] < (peer + 1) * local)).any())
         if fault == FAULT_NO_COUNTS_READY:
@@ -217,11 +216,7 @@ def test_random_configurations_with_a_faulty_peer():
         else:
             expected = 18 if peer_sends else 0
         print(f"case {case}: {c} peer={peer} fault={fault} expected code {expected}", flush=True)
-        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=300,
-                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
-                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
-        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=topk, num_experts=experts, config=config,
-                                num_ranks=world, rank=me, tx_waves=c["waves"][0], rx_waves=c["waves"][1], worker_groups=c["waves"][2]) as buffer:
+        with walk_buffer(c, timeout_ms=300) as buffer:
             buffer.peers.inject_fault(peer, fault)
             for source, (x, idx, weights) in enumerate(inputs):
                 if source != me:

@@ -44,23 +44,32 @@ def draw(case: int) -> dict:
     )
 
 
+def walk_buffer(c: dict, buffer_options: dict | None = None, **config):
+    """The buffer of a drawn configuration; ``config`` overrides fields of its HostStagedConfig."""
+    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
+
+    fields = dict(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
+                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
+                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
+    fields.update(config)
+    return HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
+                              config=HostStagedConfig(**fields), num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0],
+                              rx_waves=c["waves"][1], worker_groups=c["waves"][2], **(buffer_options or {}))
+
+
+def walk_inputs(c: dict, seed: int):
+    return make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=seed, gaussian=c["fp8"], heavy_tail=c["fp8"])
+
+
 # 1180-1199: among them a stand-alone expand whose grid is wider than its pool of ten rows.
 @pytest.mark.parametrize("first", list(range(0, 120, 20)) + [1180])
 def test_random_configurations(first):
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
-
     for case in range(first, first + 20):
         c = draw(case)
         print(f"case {case}: {c}", flush=True)
-        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
-                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
-                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
-        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
-                                config=config, num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0], rx_waves=c["waves"][1],
-                                worker_groups=c["waves"][2]) as buffer:
+        with walk_buffer(c) as buffer:
             for repeat in range(2):
-                inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + repeat,
-                                     gaussian=c["fp8"], heavy_tail=c["fp8"])
+                inputs = walk_inputs(c, case * 10 + repeat)
                 capture = c["world"] > 1
                 result, _ = run_dispatch(buffer, inputs, expand=c["expand"], alignment=c["alignment"], zero_padding=c["expand"],
                                          with_weights=c["weights"], capture=capture)
@@ -77,8 +86,6 @@ def test_random_configurations_through_the_relay(first):
     """The same walk in NUMA relay mode (stage 8): a random map of the ranks onto
     two to four NUMA domains and random replica ring sizes, so rows cross domains
     in both directions through relay workers and replica rings of every shape."""
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
-
     for case in range(first, first + 20):
         c = draw(case)
         if c["world"] == 1:
@@ -90,15 +97,9 @@ def test_random_configurations_through_the_relay(first):
             nodes = tuple(index % 2 for index in range(c["world"]))
         replica_slots = rng.choice([1, 2, 4, 16])
         print(f"case {case}: {c} nodes={nodes} replica_slots={replica_slots}", flush=True)
-        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000, stage=8,
-                                  numa_mode="relay", replica_slots=replica_slots, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16",
-                                  fuse_receive_expand=c["fuse"], receive_expand_mode="pipelined" if c["fuse"] else "scalar")
-        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
-                                config=config, num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0], rx_waves=c["waves"][1],
-                                worker_groups=c["waves"][2], rank_numa_nodes=nodes) as buffer:
+        with walk_buffer(c, {"rank_numa_nodes": nodes}, stage=8, numa_mode="relay", replica_slots=replica_slots) as buffer:
             for repeat in range(2):
-                inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + repeat,
-                                     gaussian=c["fp8"], heavy_tail=c["fp8"])
+                inputs = walk_inputs(c, case * 10 + repeat)
                 result, _ = run_dispatch(buffer, inputs, expand=c["expand"], alignment=c["alignment"], zero_padding=c["expand"],
                                          with_weights=c["weights"], capture=True)
                 verify_dispatch(result, inputs, c["rank"], c["world"], c["experts"], c["topk"], c["expand"], c["alignment"], c["expand"],
@@ -115,28 +116,20 @@ def test_random_configurations_through_cached_layouts_and_graphs(first):
     fresh payload and weights on every rank, fresh routes on the other ranks and -
     where the graph recomputes them - on the own rank, and an eager dispatch between
     the replays; three cases in ten run the prologue as a launch of its own."""
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
-
     for case in range(first, first + 20):
         c = draw(case)
         rng = random.Random(case * 13 + 5)
         split = rng.random() < 0.3
         mode = rng.choice(["dynamic", "static", "cached"])
         print(f"case {case}: {c} split_launch={split} mode={mode}", flush=True)
-        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
-                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
-                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar", enable_graph=True)
         me, expand, weighted = c["rank"], c["expand"], c["weights"]
 
         def check(result, inputs):
             verify_dispatch(result, inputs, me, c["world"], c["experts"], c["topk"], expand, c["alignment"], expand, with_weights=weighted,
                             fp8_wire=c["fp8"])
 
-        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
-                                config=config, num_ranks=c["world"], rank=me, tx_waves=c["waves"][0], rx_waves=c["waves"][1],
-                                worker_groups=c["waves"][2], split_launch=split) as buffer:
-            inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10,
-                                 gaussian=c["fp8"], heavy_tail=c["fp8"])
+        with walk_buffer(c, {"split_launch": split}, enable_graph=True) as buffer:
+            inputs = walk_inputs(c, case * 10)
             result, (x, idx, weights) = run_dispatch(buffer, inputs, expand=expand, alignment=c["alignment"], zero_padding=expand,
                                                      with_weights=weighted)
             check(result, inputs)
@@ -149,8 +142,7 @@ def test_random_configurations_through_cached_layouts_and_graphs(first):
             elif mode == "static":
                 graph = buffer.capture_dispatch(x, topk_weights=own_weights, handle=cache, do_expand=expand, do_zero_padding=expand)
             for step in range(3):
-                fresh = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + 1 + step,
-                                    gaussian=c["fp8"], heavy_tail=c["fp8"])
+                fresh = walk_inputs(c, case * 10 + 1 + step)
                 x.copy_(fresh[me][0])
                 weights.copy_(fresh[me][2])
                 if mode == "dynamic":

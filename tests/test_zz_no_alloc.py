@@ -130,22 +130,15 @@ def test_static_scratch_random_configurations():
     point, two dispatches each: consecutive runtimes of every shape (world size,
     channels, ring sizes, wavefront counts, both wires, both layouts) find each
     other's leftovers in the one array."""
-    from pcie_ep import HostStagedConfig, HostStagedEPBuffer
-    from test_gpu_random_configs import draw
+    from test_gpu_random_configs import draw, walk_buffer, walk_inputs
 
     for case in range(5000, 5040):
         c = draw(case)
         print(f"  case {case}: {c}", flush=True)
-        config = HostStagedConfig(channels=c["channels"], payload_slots=c["slots"], descriptor_slots=c["descriptors"], timeout_ms=8000,
-                                  stage=7 if c["fp8"] else 6, wire_dtype="fp8_e4m3" if c["fp8"] else "bf16", fuse_receive_expand=c["fuse"],
-                                  receive_expand_mode="pipelined" if c["fuse"] else "scalar")
-        with HostStagedEPBuffer(num_max_tokens_per_rank=c["tmax"], hidden=c["hidden"], num_topk=c["topk"], num_experts=c["experts"],
-                                config=config, num_ranks=c["world"], rank=c["rank"], tx_waves=c["waves"][0], rx_waves=c["waves"][1],
-                                worker_groups=c["waves"][2]) as buffer:
+        with walk_buffer(c) as buffer:
             buffer.runtime.use_static_scratch = True
             for repeat in range(2):
-                inputs = make_inputs(c["world"], c["tokens"], c["hidden"], c["experts"], c["topk"], c["pattern"], seed=case * 10 + repeat,
-                                     gaussian=c["fp8"], heavy_tail=c["fp8"])
+                inputs = walk_inputs(c, case * 10 + repeat)
                 result, _ = run_dispatch(buffer, inputs, expand=c["expand"], alignment=c["alignment"], zero_padding=c["expand"],
                                          with_weights=c["weights"], capture=c["world"] > 1)
                 verify_dispatch(result, inputs, c["rank"], c["world"], c["experts"], c["topk"], c["expand"], c["alignment"], c["expand"],
