@@ -108,6 +108,35 @@ def test_four_runtimes_with_the_prologue_as_a_launch_of_its_own():
         run_world(4, [33, 64, 0, 17], 512, 4, 32, ROUNDS[:3], channels=2, payload_slots=3, descriptor_slots=2, worker_groups=4, split_launch=split)
 
 
+def draw_world(rng):
+    """A random world of two to four runtimes: (world, experts per rank, experts, top-k, row length, tokens per rank, FP8 wire, configuration)."""
+    world = rng.choice([2, 2, 3, 4])
+    local = rng.choice([1, 2, 4, 8, 16])
+    experts = world * local
+    topk = rng.randint(1, min(8, experts))
+    hidden = rng.choice([8, 64, 129, 512, 1024, 2048, 7168])
+    tmax = rng.choice([1, 5, 33, 64, 96, 200])
+    tokens = [rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)]
+    if max(tokens) == 0:
+        tokens[0] = 1
+    fp8 = rng.random() < 0.3
+    config = dict(channels=rng.randint(1, 4), payload_slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptor_slots=rng.choice([1, 2, 3, 5, 16, 256]),
+                  worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3)
+    if fp8:
+        config.update(stage=7, wire_dtype="fp8_e4m3")
+    return world, local, experts, topk, hidden, tokens, fp8, config
+
+
+def draw_domains(rng, world, config):
+    """Deals the ranks onto two to four NUMA domains and switches `config` to relay mode; returns the map."""
+    domains = rng.randint(2, min(4, world))
+    nodes = tuple(rng.randrange(domains) for _ in range(world))
+    if len(set(nodes)) < 2:
+        nodes = tuple(index % 2 for index in range(world))
+    config.update(stage=8, numa_mode="relay", replica_slots=rng.choice([1, 2, 4, 16]), rank_numa_nodes=nodes)
+    return nodes
+
+
 @pytest.mark.parametrize("relay", [False, True], ids=["direct", "relay"])
 def test_random_worlds_of_runtimes(relay):
     """A seeded walk over worlds of two to four runtimes: world size, ragged and
@@ -122,26 +151,9 @@ def test_random_worlds_of_runtimes(relay):
 
     for case in range(40 if relay else 60):
         rng = random.Random(case * 31 + 7)
-        world = rng.choice([2, 2, 3, 4])
-        local = rng.choice([1, 2, 4, 8, 16])
-        experts = world * local
-        topk = rng.randint(1, min(8, experts))
-        hidden = rng.choice([8, 64, 129, 512, 1024, 2048, 7168])
-        tmax = rng.choice([1, 5, 33, 64, 96, 200])
-        tokens = [rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)]
-        if max(tokens) == 0:
-            tokens[0] = 1
-        fp8 = rng.random() < 0.3
-        config = dict(channels=rng.randint(1, 4), payload_slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptor_slots=rng.choice([1, 2, 3, 5, 16, 256]),
-                      worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3)
-        if fp8:
-            config.update(stage=7, wire_dtype="fp8_e4m3")
+        world, local, experts, topk, hidden, tokens, fp8, config = draw_world(rng)
         if relay:
-            domains = rng.randint(2, min(4, world))
-            nodes = tuple(rng.randrange(domains) for _ in range(world))
-            if len(set(nodes)) < 2:
-                nodes = tuple(index % 2 for index in range(world))
-            config.update(stage=8, numa_mode="relay", replica_slots=rng.choice([1, 2, 4, 16]), rank_numa_nodes=nodes)
+            draw_domains(rng, world, config)
         rounds = []
         for _ in range(rng.randint(2, 4)):
             pattern = rng.choice(["random", "random", "multicast", "hotspot", "local", "none", "partial"])
@@ -167,27 +179,9 @@ def test_worlds_of_runtimes_replaying_captured_dispatches():
         CALLER = torch.cuda.Stream()
     for case in range(30):
         rng = random.Random(case * 37 + 11)
-        world = rng.choice([2, 2, 3, 4])
-        local = rng.choice([1, 2, 4, 8, 16])
-        experts = world * local
-        topk = rng.randint(1, min(8, experts))
-        hidden = rng.choice([8, 64, 129, 512, 1024, 2048, 7168])
-        tmax = rng.choice([1, 5, 33, 64, 96, 200])
-        tokens = [rng.choice([0, 1, tmax, rng.randint(0, tmax)]) for _ in range(world)]
-        if max(tokens) == 0:
-            tokens[0] = 1
-        fp8 = rng.random() < 0.3
-        config = dict(channels=rng.randint(1, 4), payload_slots=rng.choice([1, 2, 3, 5, 16, 256]), descriptor_slots=rng.choice([1, 2, 3, 5, 16, 256]),
-                      worker_groups=rng.choice([2, 4, 8]), split_launch=rng.random() < 0.3, enable_graph=True)
-        if fp8:
-            config.update(stage=7, wire_dtype="fp8_e4m3")
-        nodes = None
-        if rng.random() < 0.3:
-            domains = rng.randint(2, min(4, world))
-            nodes = tuple(rng.randrange(domains) for _ in range(world))
-            if len(set(nodes)) < 2:
-                nodes = tuple(index % 2 for index in range(world))
-            config.update(stage=8, numa_mode="relay", replica_slots=rng.choice([1, 2, 4, 16]), rank_numa_nodes=nodes)
+        world, local, experts, topk, hidden, tokens, fp8, config = draw_world(rng)
+        config["enable_graph"] = True
+        nodes = draw_domains(rng, world, config) if rng.random() < 0.3 else None
         expand = rng.random() < 0.7
         alignment = rng.choice([1, 2, 8, 16, 128]) if expand else 1
         weighted = rng.random() < 0.8
